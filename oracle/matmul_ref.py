@@ -1,0 +1,109 @@
+"""CPU oracle: grouped matmul, SwiGLU and the top-k combine.  Test infrastructure, never shipped.
+
+Restates, with torch-CPU float32 arithmetic:
+  matmul_ref   matmul.py:823-914 (matmul_torch) + :755-800 (apply_precision)
+  swiglu_ref   swiglu.py:89-100 (swiglu_torch)
+  reduce_ref   reduce.py:1173-1206 (reduce_torch), sum/mask/scale part
+"""
+import torch
+
+from .mxfp_ref import upcast_from_mxfp_ref
+
+
+def dequant_operand(t: torch.Tensor, mx_scale, flex_scale, mx_axis: int):
+    """apply_precision (matmul.py:755-800): an mx operand is dequantised to
+    bfloat16 (:772-778, 788-794); a flex (per-tensor scaled fp8) operand becomes
+    float32 value*scale (:761-764); anything else is used as is."""
+    if mx_scale is not None:
+        return upcast_from_mxfp_ref(t, mx_scale, torch.bfloat16, axis=mx_axis)
+    if flex_scale is not None:
+        return t.to(torch.float32) * flex_scale.to(torch.float32)
+    return t.clone()
+
+
+def matmul_ref(a, b, bias, slice_sizes=None, gather_indx=None, scatter_indx=None,
+               a_mx_scale=None, b_mx_scale=None, a_flex_scale=None, b_flex_scale=None,
+               betas=None, gammas=None, out_scale=None, out_alpha=None, fused_swiglu=None):
+    """y[rows of slice e] = (a[gather] @ deq(b[e])) + bias[e]*beta, times gamma,
+    computed in float32 and stored in the dtype of the dequantised `a`
+    (matmul.py:887-902); rows are then placed at scatter_indx (-1 drops the row,
+    :905-910); the result is divided by out_scale when given (:914).
+
+    fused_swiglu=(alpha, limit) applies the activation to the float32 result
+    before gamma and before the cast, the order of the reference's GPU kernel
+    (matmul_details/_matmul.py:540-559); without it the caller applies
+    swiglu_ref to the rounded output, the order of the reference's test
+    (tests/test_matmul.py:599-600).  out_alpha multiplies after the bias (:548-550).
+
+    a: [M, K] (or [B, M, K] batched); b: [E, K, N] / [K, N], mxfp4 weights as
+    packed uint8 [E, K/2, N] with b_mx_scale uint8 [E, K/32, N].
+    slice_sizes: int32 [E] rows per expert in expert-sorted order (ragged M).
+    """
+    a = dequant_operand(a, a_mx_scale, a_flex_scale, a.ndim - 1)
+    b = dequant_operand(b, b_mx_scale, b_flex_scale, b.ndim - 2)
+    batched = a.ndim == 3
+    if bias is not None and bias.ndim == 1:
+        bias = bias[None]
+    if b.ndim == 2:
+        b = b[None]
+    if a.ndim == 2:
+        a = a[None]
+    if slice_sizes is not None and not batched:
+        offs = [0]
+        for s in slice_sizes.tolist():
+            offs.append(offs[-1] + int(s))
+        spans = list(zip(offs[:-1], offs[1:]))
+    else:
+        spans = [(0, a.shape[1])] * b.shape[0]
+    n_rows = a.shape[1] if gather_indx is None else gather_indx.shape[0]
+    n_out = b.shape[-1] // 2 if fused_swiglu is not None else b.shape[-1]
+    y = torch.zeros((a.shape[0], n_rows, n_out), dtype=a.dtype)
+    for e, (lo, hi) in enumerate(spans):
+        rows = torch.arange(lo, hi) if gather_indx is None else gather_indx[lo:hi].long()
+        z = e if batched else 0
+        out = a[z, rows, :].to(torch.float32) @ b[e].to(torch.float32)
+        if bias is not None:
+            bb = bias[e].to(torch.float32)
+            out = out + (bb if betas is None else bb * betas[lo:hi, None].to(torch.float32))
+        if out_alpha is not None:
+            out = out * out_alpha
+        if fused_swiglu is not None:
+            out = swiglu_ref(out, fused_swiglu[0], fused_swiglu[1])
+        if gammas is not None:
+            out = out * gammas[lo:hi, None].to(torch.float32)
+        y[z, lo:hi, :] = out.to(y.dtype)
+    if not batched:
+        y = y[0]
+    if scatter_indx is not None:
+        out = torch.zeros((scatter_indx.shape[0], y.shape[-1]), dtype=y.dtype)
+        keep = scatter_indx != -1
+        out[scatter_indx[keep].long()] = y[keep]
+        y = out
+    if out_scale is not None:
+        y = y / out_scale
+    return y
+
+
+def swiglu_ref(a: torch.Tensor, alpha: float, limit):
+    """Interleaved SwiGLU, swiglu.py:89-100: gate = even columns clamped from
+    above, linear = odd columns clamped to [-limit, limit];
+    out = gate*sigmoid(alpha*gate) * (linear + 1), evaluated in float32."""
+    dt = a.dtype
+    a = a.to(torch.float32)
+    g = a[..., 0::2]
+    l = a[..., 1::2]
+    if limit is not None:
+        g = g.clamp(max=limit)
+        l = l.clamp(min=-limit, max=limit)
+    return ((g * torch.sigmoid(alpha * g)) * (l + 1)).to(dt)
+
+
+def reduce_ref(x: torch.Tensor, dim: int, mask=None, scale=None):
+    """sum over `dim` of where(mask, x*scale, 0) in float32, cast back to
+    x.dtype; reduce.py:1179-1206 without the mx / flex branches."""
+    xf = x.to(torch.float32)
+    if scale is not None:
+        xf = xf * scale.to(torch.float32)
+    if mask is not None:
+        xf = torch.where(mask.to(torch.bool), xf, torch.zeros((), dtype=torch.float32))
+    return xf.sum(dim=dim).to(x.dtype)

@@ -1,0 +1,49 @@
+"""GPU parity: top-k combine (reduce) and standalone SwiGLU vs the CPU oracle."""
+import pytest
+import torch
+
+from oracle import matmul_ref as MR
+from triton_amd.reduce import reduce
+from triton_amd.swiglu import PrecisionConfig, swiglu
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,dim", [((512, 4, 2880), 1), ((4, 300, 64), 0), ((37, 5, 33), 1), ((8, 16), 1), ((6, 7, 8), 2)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("mask_mode", [None, "full", "broadcast_last"])
+def test_reduce(shape, dim, dtype, mask_mode, device):
+    torch.manual_seed(0)
+    x = torch.randn(shape).to(dtype)
+    mask = None
+    if mask_mode == "full":
+        mask = torch.rand(shape) > 0.3
+    elif mask_mode == "broadcast_last":
+        mshape = list(shape)
+        mshape[-1] = 1
+        mask = torch.rand(mshape) > 0.3
+    y, _ = reduce(x.to(device), dim, mask=None if mask is None else mask.to(device))
+    ref = MR.reduce_ref(x, dim, mask=mask)
+    tol = dict(rtol=1e-2, atol=1e-2) if dtype != torch.float32 else dict(rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(y.cpu().float(), ref.float(), **tol)
+
+
+def test_reduce_scale(device):
+    torch.manual_seed(1)
+    x = torch.randn(64, 4, 256).to(torch.bfloat16)
+    scale = torch.rand(64, 4, 1)
+    y, _ = reduce(x.to(device), 1, scale=scale.to(device))
+    ref = MR.reduce_ref(x, 1, scale=scale)
+    torch.testing.assert_close(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N", [(1311, 4352), (7, 30)])
+@pytest.mark.parametrize("limit", [1e-2, 10.0, None])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_swiglu(M, N, limit, dtype, device):
+    torch.manual_seed(2)
+    x = torch.randn(M, N).to(dtype)
+    out = swiglu(x.to(device), 0.5, PrecisionConfig(limit))
+    ref = MR.swiglu_ref(x, 0.5, limit)
+    tol = dict(rtol=1e-2, atol=1e-2) if dtype != torch.float32 else dict(rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), **tol)

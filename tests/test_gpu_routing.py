@@ -1,0 +1,119 @@
+"""GPU parity: topk, bitmatrix metadata, ragged metadata and routing() vs the CPU oracle (bit-exact integers)."""
+import pytest
+import torch
+
+from oracle import routing_ref as R
+from triton_amd.routing import routing
+from triton_amd.tensor import BIT, make_bitmatrix_metadata, make_ragged_tensor_metadata, wrap_torch_tensor
+from triton_amd.topk import topk
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n_rows", [1, 7, 256, 300])
+@pytest.mark.parametrize("n_cols", [13, 32, 128, 200, 811])
+@pytest.mark.parametrize("k", [1, 4, 8])
+@pytest.mark.parametrize("apply_softmax", [True, False])
+def test_topk(n_rows, n_cols, k, apply_softmax, device):
+    torch.manual_seed(0)
+    x = torch.randn(n_rows, n_cols)
+    sp = topk(x.to(device), k, apply_softmax=apply_softmax)
+    vals, indx, bits = R.topk_ref(x, k, apply_softmax)
+    assert sp.indx.dtype == torch.int16
+    assert torch.equal(sp.indx.cpu().int(), indx)
+    torch.testing.assert_close(sp.vals.cpu(), vals, rtol=1e-5, atol=1e-6)
+    store = sp.mask.storage.data
+    assert store.stride() == (1, -(-n_rows // 32) * 32) and tuple(store.shape) == (n_rows, -(-n_cols // 32))
+    assert torch.equal(store.cpu().view(torch.int32), bits)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_topk_ties_and_16bit(dtype, device):
+    torch.manual_seed(1)
+    x = torch.randn(300, 128).to(dtype)  # 16-bit logits collide often: exercises the lower-index-wins rule
+    x[:, 64:] = x[:, :64]
+    sp = topk(x.to(device), 4)
+    vals, indx, bits = R.topk_ref(x, 4)
+    assert torch.equal(sp.indx.cpu().int(), indx)
+    assert torch.equal(sp.mask.storage.data.cpu().view(torch.int32), bits)
+    torch.testing.assert_close(sp.vals.cpu().float(), vals.float(), rtol=2e-2, atol=1e-3)
+
+
+def test_topk_n_rows_and_provided_indx(device):
+    torch.manual_seed(2)
+    x = torch.randn(100, 64)
+    sp = topk(x.to(device), 4, n_rows=70)
+    vals, indx, bits = R.topk_ref(x, 4, n_rows=70)
+    assert torch.equal(sp.indx.cpu().int()[:70], indx[:70])
+    assert torch.equal(sp.mask.storage.data.cpu().view(torch.int32)[:70], bits[:70])
+    y_indx = torch.stack([torch.randperm(64)[:4] for _ in range(100)]).to(torch.int16)
+    sp = topk(x.to(device), 4, y_indx=y_indx.to(device))
+    vals, indx, bits = R.topk_ref(x, 4, y_indx=y_indx)
+    torch.testing.assert_close(sp.vals.cpu(), vals, rtol=1e-5, atol=1e-6)
+    assert torch.equal(sp.mask.storage.data.cpu().view(torch.int32), bits)
+
+
+@pytest.mark.parametrize("n_rows", [7, 256, 17111])
+@pytest.mark.parametrize("n_cols", [13, 32, 128, 811])
+@pytest.mark.parametrize("k", [1, 4, 8])
+def test_bitmatrix_metadata(n_rows, n_cols, k, device):
+    torch.manual_seed(0)
+    indx = torch.rand(n_rows, n_cols).argsort(dim=1).int()[:, :k]
+    indx = torch.sort(indx, dim=1)[0]
+    bm = wrap_torch_tensor(torch.zeros((n_rows, (n_cols + 31) // 32), dtype=torch.int32, device=device).view(torch.uint32),
+                           dtype=BIT, shape=(n_rows, n_cols))
+    m = make_bitmatrix_metadata(indx.to(device), bm)
+    ref = R.bitmatrix_metadata_ref(indx, n_cols)
+    assert torch.equal(m.col_sum.cpu(), ref.col_sum)
+    assert torch.equal(m.row_sorted_indx.cpu(), ref.row_sorted_indx)
+    assert torch.equal(m.col_sorted_indx.cpu(), ref.col_sorted_indx)
+
+
+def test_bitmatrix_metadata_with_dropped_rows(device):
+    torch.manual_seed(3)
+    indx = torch.randint(0, 40, (500, 4), dtype=torch.int32)
+    indx[350:] = -1
+    bm = wrap_torch_tensor(torch.zeros((500, 2), dtype=torch.int32, device=device).view(torch.uint32), dtype=BIT,
+                           shape=(500, 40))
+    m = make_bitmatrix_metadata(indx.to(device), bm)
+    ref = R.bitmatrix_metadata_ref(indx, 40)
+    assert torch.equal(m.col_sum.cpu(), ref.col_sum)
+    assert torch.equal(m.row_sorted_indx.cpu(), ref.row_sorted_indx)
+    assert torch.equal(m.col_sorted_indx.cpu(), ref.col_sorted_indx)
+
+
+@pytest.mark.parametrize("n_slices", [1, 7, 33, 911, 1025])
+def test_ragged_metadata(n_slices, device):
+    torch.manual_seed(0)
+    max_slice = 200
+    total = max_slice * n_slices
+    sizes = torch.randint(0, max_slice, (n_slices, ), dtype=torch.int32)
+    sizes[torch.randint(0, n_slices, (1, ))] = 0
+    m = make_ragged_tensor_metadata(sizes.to(device), total)
+    ref = R.ragged_metadata_ref(sizes, total)
+    assert torch.equal(m.slice_offs.cpu(), ref.slice_offs)
+    assert torch.equal(m.block_offs_data.cpu(), ref.block_offs_data)
+    assert torch.equal(m.block_schedule_data.cpu(), ref.block_schedule_data)
+
+
+@pytest.mark.parametrize("T,E,k", [(4096, 128, 4), (64, 128, 4), (16384, 32, 4), (300, 200, 8), (1, 128, 4)])
+def test_routing_configs(T, E, k, device):
+    """BASELINE config 2 (T=4096, E=128, k=4) and the routing of configs 4 / 5, plus a run with exact ties."""
+    torch.manual_seed(0)
+    for ties in (False, True):
+        logits = torch.randn(T, E)
+        if ties:
+            logits[:, E // 2:E // 2 * 2] = logits[:, :E // 2]
+        out = routing(logits.to(device), k)
+        ref = R.routing_ref(logits, k)
+        assert torch.equal(out.indx.cpu().int(), ref["indx"])
+        assert torch.equal(out.col_sum.cpu(), ref["col_sum"])
+        assert torch.equal(out.scatter_indx.cpu(), ref["scatter_indx"])
+        assert torch.equal(out.row_sorted_indx.cpu(), ref["row_sorted_indx"])
+        assert torch.equal(out.gather_indx.cpu(), ref["gather_indx"])
+        rm = out.ragged_metadata
+        assert torch.equal(rm.slice_offs.cpu(), ref["ragged"].slice_offs)
+        assert torch.equal(rm.block_offs_data.cpu(), ref["ragged"].block_offs_data)
+        assert torch.equal(rm.block_schedule_data.cpu(), ref["ragged"].block_schedule_data)
+        torch.testing.assert_close(out.vals.cpu(), ref["vals"], rtol=1e-5, atol=1e-6)
+        assert int(out.col_sum.sum()) == T * k

@@ -1,0 +1,85 @@
+// Shared device / host helpers for the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/triton_amd.h"
+
+#define TAMD_DEVICE __device__ __forceinline__
+
+namespace tamd {
+
+constexpr int kWave = 64;
+
+TAMD_DEVICE float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+TAMD_DEVICE uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+TAMD_DEVICE float bf16_bits_to_f32(uint32_t h) { return bits_to_f32(h << 16); }
+
+// float32 -> bfloat16 bits, round to nearest even, NaN kept quiet.
+TAMD_DEVICE uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = f32_to_bits(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+TAMD_DEVICE float f16_bits_to_f32(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+TAMD_DEVICE uint32_t f32_to_f16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// OCP e4m3fn byte -> float32 (exact).
+TAMD_DEVICE float e4m3_bits_to_f32(uint32_t b) {
+  uint32_t s = (b & 0x80u) << 24;
+  uint32_t e = (b >> 3) & 0xFu;
+  uint32_t m = b & 7u;
+  float mag;
+  if (e == 0) {
+    mag = (float)m * 0.001953125f;  // m * 2^-9
+  } else if (e == 15 && m == 7) {
+    mag = bits_to_f32(0x7FC00000u);
+  } else {
+    mag = bits_to_f32(((e + 120u) << 23) | (m << 20));
+  }
+  return bits_to_f32(f32_to_bits(mag) | s);
+}
+
+template <int DT>
+TAMD_DEVICE float load_as_f32(const void *p, int64_t i) {
+  if constexpr (DT == TAMD_F32) return ((const float *)p)[i];
+  if constexpr (DT == TAMD_BF16) return bf16_bits_to_f32(((const uint16_t *)p)[i]);
+  if constexpr (DT == TAMD_F16) return f16_bits_to_f32(((const uint16_t *)p)[i]);
+  if constexpr (DT == TAMD_FP8_E4M3) return e4m3_bits_to_f32(((const uint8_t *)p)[i]);
+  return 0.f;
+}
+
+template <int DT>
+TAMD_DEVICE void store_from_f32(void *p, int64_t i, float v) {
+  if constexpr (DT == TAMD_F32) ((float *)p)[i] = v;
+  if constexpr (DT == TAMD_BF16) ((uint16_t *)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+  if constexpr (DT == TAMD_F16) ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v);
+}
+
+inline int dtype_size(int dt) {
+  switch (dt) {
+    case TAMD_F32: return 4;
+    case TAMD_F16:
+    case TAMD_BF16: return 2;
+    case TAMD_FP8_E4M3:
+    case TAMD_FP8_E5M2:
+    case TAMD_MXFP4: return 1;
+    default: return 0;
+  }
+}
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // namespace tamd

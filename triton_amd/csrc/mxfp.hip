@@ -1,0 +1,389 @@
+// MXFP4 quantise / dequantise for gfx950.  Bandwidth kernels: 128-bit global
+// accesses, one 32-element group handled by 4 lanes (quantised axis contiguous)
+// or by one lane per column (quantised axis strided, i.e. the weight layout).
+//
+// Arithmetic follows numerics_details/mxfp.py:212-363 and :384-449 of the
+// reference: scale = 2^ceil(log2(max/6)) taken from the float32 bit pattern,
+// q = x * (1/scale), round-to-nearest-even onto {0,.5,1,1.5,2,3,4,6}, saturate.
+#include "common.h"
+
+namespace tamd {
+
+// e2m1 code (sign in bit 3) of q: nearest grid value, ties to the even code.
+TAMD_DEVICE uint32_t e2m1_code(float q) {
+  float a = __builtin_fabsf(q);
+  uint32_t c = (uint32_t)(a > 0.25f) + (uint32_t)(a >= 0.75f) + (uint32_t)(a > 1.25f) +
+               (uint32_t)(a >= 1.75f) + (uint32_t)(a > 2.5f) + (uint32_t)(a >= 3.5f) +
+               (uint32_t)(a > 5.0f);
+  if (a != a) c = 7u;
+  return c | ((f32_to_bits(q) >> 28) & 8u);
+}
+
+// Returns the multiplier 1/scale and writes the e8m0 byte.
+TAMD_DEVICE float group_scale(float gmax, int mode, uint32_t &scale_byte) {
+  uint32_t sb;
+  if (mode == TAMD_ROUND_UP) {
+    sb = (f32_to_bits(gmax / 6.0f) + 0x007FFFFFu) & 0x7F800000u;
+  } else {
+    sb = f32_to_bits(gmax * 0.25f) & 0x7F800000u;
+  }
+  scale_byte = sb >> 23;
+  float ds = bits_to_f32(sb);
+  return ds == 0.f ? 0.f : 1.0f / ds;
+}
+
+TAMD_DEVICE float e2m1_value(uint32_t code) {
+  uint32_t m = code & 7u;
+  uint32_t bits = m < 2u ? (m ? 0x3F000000u : 0u) : ((((m >> 1) + 126u) << 23) | ((m & 1u) << 22));
+  return bits_to_f32(bits | ((code & 8u) << 28));
+}
+
+template <int DT>
+constexpr float kMaxFinite =
+    DT == TAMD_F32 ? 3.4028234663852886e+38f : (DT == TAMD_BF16 ? 3.3895313892515355e+38f : 65504.f);
+
+template <int DT>
+TAMD_DEVICE float dequant_one(uint32_t code, float mult, bool is_nan) {
+  float v = e2m1_value(code) * mult;
+  constexpr float mf = kMaxFinite<DT>;
+  v = v != v ? v : __builtin_fminf(__builtin_fmaxf(v, -mf), mf);
+  return is_nan ? bits_to_f32(0x7FC00000u) : v;
+}
+
+template <int DT>
+TAMD_DEVICE uint32_t pack2(float a, float b) {
+  if constexpr (DT == TAMD_BF16) return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+  return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+}
+
+// ---------------------------------------------------------------------------
+// downcast, quantised axis contiguous in the source: 4 lanes x 8 elements per group
+// ---------------------------------------------------------------------------
+template <int DT, bool VEC>
+__global__ __launch_bounds__(256) void downcast_rows_kernel(
+    const void *__restrict__ src, int64_t n_groups_total, int64_t G, int64_t nr, int64_t ssb, int64_t ssr,
+    uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
+    int64_t csr, int mode) {
+  int64_t gid = (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);
+  int sub = threadIdx.x & 3;
+  bool live = gid < n_groups_total;
+  int64_t gg = live ? gid : 0;
+  int64_t run = gg / G, g = gg - run * G;
+  int64_t b = run / nr, r = run - b * nr;
+  int64_t off = b * ssb + r * ssr + g * 32 + sub * 8;
+  float v[8];
+  if constexpr (VEC && DT == TAMD_F32) {
+    const float4 *p = (const float4 *)((const float *)src + off);
+    float4 a = p[0], c = p[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = c.x; v[5] = c.y; v[6] = c.z; v[7] = c.w;
+  } else if constexpr (VEC) {
+    uint4 a = *(const uint4 *)((const uint16_t *)src + off);
+    uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (DT == TAMD_BF16) {
+        v[2 * j] = bf16_bits_to_f32(w[j] & 0xFFFFu);
+        v[2 * j + 1] = bf16_bits_to_f32(w[j] >> 16);
+      } else {
+        v[2 * j] = f16_bits_to_f32(w[j] & 0xFFFFu);
+        v[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = load_as_f32<DT>(src, off + j);
+  }
+  float m = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) m = __builtin_fmaxf(m, __builtin_fabsf(v[j]));
+  m = __builtin_fmaxf(m, __shfl_xor(m, 1));
+  m = __builtin_fmaxf(m, __shfl_xor(m, 2));
+  uint32_t sbyte;
+  float qs = group_scale(m, mode, sbyte);
+  uint32_t packed = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] * qs) << (4 * j);
+  if (!live) return;
+  *(uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4) = packed;
+  if (sub == 0) scales[b * csb + r * csr + g] = (uint8_t)sbyte;
+}
+
+// ---------------------------------------------------------------------------
+// downcast, source contiguous along r (quantised axis strided): a thread owns
+// NV adjacent columns and walks the 32 rows of one group, keeping them in registers.
+// ---------------------------------------------------------------------------
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void downcast_cols_kernel(
+    const void *__restrict__ src, int64_t nb, int64_t G, int64_t nr, int64_t ssb, int64_t ssl,
+    uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
+    int64_t csr, int mode) {
+  int64_t n_rv = (nr + NV - 1) / NV;
+  int64_t blocks_r = (n_rv + 255) / 256;
+  int64_t bid = blockIdx.x;
+  int64_t br = bid % blocks_r;
+  int64_t t = bid / blocks_r;
+  int64_t g = t % G;
+  int64_t b = t / G;
+  int64_t rv = br * 256 + threadIdx.x;
+  if (rv >= n_rv) return;
+  int64_t r0 = rv * NV;
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  const char *base = (const char *)src + (b * ssb + g * 32 * ssl + r0) * ES;
+  float mx[NV];
+#pragma unroll
+  for (int c = 0; c < NV; ++c) mx[c] = 0.f;
+  if constexpr (NV == 1) {
+    float v[32];
+#pragma unroll
+    for (int l = 0; l < 32; ++l) {
+      v[l] = load_as_f32<DT>(base, l * ssl);
+      mx[0] = __builtin_fmaxf(mx[0], __builtin_fabsf(v[l]));
+    }
+    uint32_t sbyte;
+    float qs = group_scale(mx[0], mode, sbyte);
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int l = 0; l < 32; ++l) w[l >> 3] |= e2m1_code(v[l] * qs) << (4 * (l & 7));
+    *(uint4 *)(vals + b * vsb + r0 * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+    scales[b * csb + r0 * csr + g] = (uint8_t)sbyte;
+  } else {
+    uint4 raw[32];
+#pragma unroll
+    for (int l = 0; l < 32; ++l) raw[l] = *(const uint4 *)(base + (int64_t)l * ssl * ES);
+    auto elem = [&](int l, int c) -> float {
+      const uint4 &q = raw[l];
+      uint32_t w[4] = {q.x, q.y, q.z, q.w};
+      if constexpr (DT == TAMD_F32) return bits_to_f32(w[c]);
+      uint32_t h = (c & 1) ? (w[c >> 1] >> 16) : (w[c >> 1] & 0xFFFFu);
+      if constexpr (DT == TAMD_BF16) return bf16_bits_to_f32(h);
+      return f16_bits_to_f32(h);
+    };
+#pragma unroll
+    for (int l = 0; l < 32; ++l)
+#pragma unroll
+      for (int c = 0; c < NV; ++c) mx[c] = __builtin_fmaxf(mx[c], __builtin_fabsf(elem(l, c)));
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      uint32_t sbyte;
+      float qs = group_scale(mx[c], mode, sbyte);
+      uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int l = 0; l < 32; ++l) w[l >> 3] |= e2m1_code(elem(l, c) * qs) << (4 * (l & 7));
+      *(uint4 *)(vals + b * vsb + (r0 + c) * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+      scales[b * csb + (r0 + c) * csr + g] = (uint8_t)sbyte;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// upcast, destination contiguous along the quantised axis
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void upcast_rows_kernel(
+    const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
+    int64_t csb, int64_t csr, void *__restrict__ dst, int64_t n_groups_total, int64_t G, int64_t nr,
+    int64_t dsb, int64_t dsr, int vec_ok) {
+  int64_t gid = (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);
+  int sub = threadIdx.x & 3;
+  if (gid >= n_groups_total) return;
+  int64_t run = gid / G, g = gid - run * G;
+  int64_t b = run / nr, r = run - b * nr;
+  uint32_t packed = *(const uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4);
+  uint32_t s = scales[b * csb + r * csr + g];
+  float mult = bits_to_f32(s << 23);
+  bool is_nan = s == 0xFFu;
+  float o[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = dequant_one<DT>((packed >> (4 * j)) & 0xFu, mult, is_nan);
+  int64_t off = b * dsb + r * dsr + g * 32 + sub * 8;
+  if (vec_ok) {
+    if constexpr (DT == TAMD_F32) {
+      float4 *p = (float4 *)((float *)dst + off);
+      p[0] = make_float4(o[0], o[1], o[2], o[3]);
+      p[1] = make_float4(o[4], o[5], o[6], o[7]);
+    } else {
+      *(uint4 *)((uint16_t *)dst + off) =
+          make_uint4(pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3]), pack2<DT>(o[4], o[5]), pack2<DT>(o[6], o[7]));
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) store_from_f32<DT>(dst, off + j, o[j]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// upcast, destination contiguous along r: a thread owns NV columns of one group
+// ---------------------------------------------------------------------------
+template <int DT, int NV>
+__global__ __launch_bounds__(256) void upcast_cols_kernel(
+    const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
+    int64_t csb, int64_t csr, void *__restrict__ dst, int64_t nb, int64_t G, int64_t nr, int64_t dsb,
+    int64_t dsl) {
+  int64_t n_rv = (nr + NV - 1) / NV;
+  int64_t blocks_r = (n_rv + 255) / 256;
+  int64_t bid = blockIdx.x;
+  int64_t br = bid % blocks_r;
+  int64_t t = bid / blocks_r;
+  int64_t g = t % G;
+  int64_t b = t / G;
+  int64_t rv = br * 256 + threadIdx.x;
+  if (rv >= n_rv) return;
+  int64_t r0 = rv * NV;
+  uint4 code[NV];
+  float mult[NV];
+  bool isn[NV];
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    code[c] = *(const uint4 *)(vals + b * vsb + (r0 + c) * vsr + g * 16);
+    uint32_t s = scales[b * csb + (r0 + c) * csr + g];
+    mult[c] = bits_to_f32(s << 23);
+    isn[c] = s == 0xFFu;
+  }
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  char *base = (char *)dst + (b * dsb + g * 32 * dsl + r0) * ES;
+#pragma unroll
+  for (int l = 0; l < 32; ++l) {
+    float o[NV];
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      uint32_t w[4] = {code[c].x, code[c].y, code[c].z, code[c].w};
+      o[c] = dequant_one<DT>((w[l >> 3] >> (4 * (l & 7))) & 0xFu, mult[c], isn[c]);
+    }
+    char *p = base + (int64_t)l * dsl * ES;
+    if constexpr (NV == 1) {
+      store_from_f32<DT>(p, 0, o[0]);
+    } else if constexpr (DT == TAMD_F32) {
+      *(float4 *)p = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+      *(uint4 *)p = make_uint4(pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3]), pack2<DT>(o[4], o[5]),
+                               pack2<DT>(o[6], o[7]));
+    }
+  }
+}
+
+template <int DT>
+int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t ssb, int64_t ssl, int64_t ssr,
+                    uint8_t *vals, int64_t vsb, int64_t vsr, uint8_t *scales, int64_t csb, int64_t csr,
+                    int mode, hipStream_t st) {
+  const int64_t G = L / 32;
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  if (ssl == 1) {
+    int64_t total = nb * nr * G;
+    bool vec = aligned(src, 16) && (ssb * ES) % 16 == 0 && (ssr * ES) % 16 == 0;
+    int64_t blocks = (total + 63) / 64;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    if (vec)
+      downcast_rows_kernel<DT, true><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
+                                                                            vsb, vsr, scales, csb, csr, mode);
+    else
+      downcast_rows_kernel<DT, false><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
+                                                                             vsb, vsr, scales, csb, csr, mode);
+    return launch_status();
+  }
+  if (ssr != 1) return TAMD_E_INVALID;
+  constexpr int NV = 16 / ES;
+  bool vec = nr % NV == 0 && aligned(src, 16) && (ssb * ES) % 16 == 0 && (ssl * ES) % 16 == 0;
+  if (vec) {
+    int64_t blocks = ((nr / NV + 255) / 256) * G * nb;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    downcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
+                                                                        scales, csb, csr, mode);
+  } else {
+    int64_t blocks = ((nr + 255) / 256) * G * nb;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    downcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
+                                                                       scales, csb, csr, mode);
+  }
+  return launch_status();
+}
+
+template <int DT>
+int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *scales, int64_t csb, int64_t csr,
+                  void *dst, int64_t nb, int64_t L, int64_t nr, int64_t dsb, int64_t dsl, int64_t dsr,
+                  hipStream_t st) {
+  const int64_t G = L / 32;
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  if (dsl == 1) {
+    int64_t total = nb * nr * G;
+    int vec = aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsr * ES) % 16 == 0;
+    int64_t blocks = (total + 63) / 64;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    upcast_rows_kernel<DT><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, total, G,
+                                                                  nr, dsb, dsr, vec);
+    return launch_status();
+  }
+  if (dsr != 1) return TAMD_E_INVALID;
+  constexpr int NV = 16 / ES;
+  bool vec = nr % NV == 0 && aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsl * ES) % 16 == 0;
+  if (vec) {
+    int64_t blocks = ((nr / NV + 255) / 256) * G * nb;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    upcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
+                                                                      nr, dsb, dsl);
+  } else {
+    int64_t blocks = ((nr + 255) / 256) * G * nb;
+    if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+    upcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
+                                                                     nr, dsb, dsl);
+  }
+  return launch_status();
+}
+
+}  // namespace tamd
+
+using namespace tamd;
+
+extern "C" int tamd_downcast_mxfp(const void *src, int src_dtype, int64_t nb, int64_t L, int64_t nr,
+                                  int64_t src_stride_b, int64_t src_stride_l, int64_t src_stride_r,
+                                  void *out_vals, int out_dtype, int64_t val_stride_b, int64_t val_stride_r,
+                                  uint8_t *out_scales, int64_t scale_stride_b, int64_t scale_stride_r,
+                                  int rounding_mode, void *stream) {
+  if (nb < 0 || L < 0 || nr < 0 || L % 32 != 0) return TAMD_E_INVALID;
+  if (rounding_mode != TAMD_ROUND_UP && rounding_mode != TAMD_ROUND_DOWN) return TAMD_E_INVALID;
+  if (out_dtype != TAMD_MXFP4) return TAMD_E_UNSUPPORTED;
+  if (nb == 0 || L == 0 || nr == 0) return 0;
+  if (!src || !out_vals || !out_scales) return TAMD_E_INVALID;
+  if (!aligned(out_vals, 16) || val_stride_b % 16 != 0 || val_stride_r % 16 != 0) return TAMD_E_ALIGNMENT;
+  hipStream_t st = (hipStream_t)stream;
+  uint8_t *v = (uint8_t *)out_vals;
+  switch (src_dtype) {
+    case TAMD_F32:
+      return launch_downcast<TAMD_F32>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
+                                       val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
+    case TAMD_BF16:
+      return launch_downcast<TAMD_BF16>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
+                                        val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
+    case TAMD_F16:
+      return launch_downcast<TAMD_F16>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
+                                       val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
+    default:
+      return TAMD_E_INVALID;
+  }
+}
+
+extern "C" int tamd_upcast_mxfp(const void *vals, int val_dtype, int64_t val_stride_b, int64_t val_stride_r,
+                                const uint8_t *scales, int64_t scale_stride_b, int64_t scale_stride_r, void *dst,
+                                int dst_dtype, int64_t nb, int64_t L, int64_t nr, int64_t dst_stride_b,
+                                int64_t dst_stride_l, int64_t dst_stride_r, void *stream) {
+  if (nb < 0 || L < 0 || nr < 0 || L % 32 != 0) return TAMD_E_INVALID;
+  if (val_dtype != TAMD_MXFP4) return TAMD_E_UNSUPPORTED;
+  if (nb == 0 || L == 0 || nr == 0) return 0;
+  if (!vals || !scales || !dst) return TAMD_E_INVALID;
+  if (!aligned(vals, 16) || val_stride_b % 16 != 0 || val_stride_r % 16 != 0) return TAMD_E_ALIGNMENT;
+  hipStream_t st = (hipStream_t)stream;
+  const uint8_t *v = (const uint8_t *)vals;
+  switch (dst_dtype) {
+    case TAMD_F32:
+      return launch_upcast<TAMD_F32>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
+                                     L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
+    case TAMD_BF16:
+      return launch_upcast<TAMD_BF16>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
+                                      L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
+    case TAMD_F16:
+      return launch_upcast<TAMD_F16>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
+                                     L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
+    default:
+      return TAMD_E_INVALID;
+  }
+}

@@ -1,0 +1,457 @@
+// Routing kernels for gfx950: top-k (+softmax, bit matrix), expert histogram with a
+// stable expert-major ordering of the (token, slot) pairs, and the ragged-tensor
+// block metadata.  Integer work only; wave64 ballots / shuffles, no float atomics,
+// results independent of scheduling.
+#include "common.h"
+
+namespace tamd {
+
+// ---------------------------------------------------------------------------
+// top-k
+// ---------------------------------------------------------------------------
+// Sort key of a logit: order-preserving map of the float32 bits in the high
+// part, (0xFFFF - column) in the low 16 bits so that the lower column wins ties
+// (topk_details/_topk_forward.py:15-30).  -0.0 is keyed as +0.0 so that both
+// zeros tie, as they do under the reference's stable argsort of -x.
+TAMD_DEVICE uint64_t logit_key(float x, int col) {
+  uint32_t u = f32_to_bits(x);
+  if (u == 0x80000000u) u = 0u;
+  u ^= (u >> 31) ? 0xFFFFFFFFu : 0x80000000u;
+  return ((uint64_t)u << 16) | (uint64_t)(0xFFFFu - (uint32_t)col);
+}
+
+template <int L>
+TAMD_DEVICE uint64_t group_max_u64(uint64_t v) {
+#pragma unroll
+  for (int o = 1; o < L; o <<= 1) {
+    uint32_t lo = __shfl_xor((uint32_t)v, o);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), o);
+    uint64_t w = ((uint64_t)hi << 32) | lo;
+    v = w > v ? w : v;
+  }
+  return v;
+}
+
+template <int L>
+TAMD_DEVICE float group_sum_f32(float v) {
+#pragma unroll
+  for (int o = 1; o < L; o <<= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+template <int L>
+TAMD_DEVICE float group_max_f32(float v) {
+#pragma unroll
+  for (int o = 1; o < L; o <<= 1) v = __builtin_fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+
+// L lanes cooperate on one row; EPL > 0 keeps ceil(n_cols/L) <= EPL keys in registers.
+template <int DT, int L, int EPL>
+__global__ __launch_bounds__(256) void topk_kernel(const void *__restrict__ x, int64_t x_stride, int n_rows,
+                                                   int n_cols, int k, int apply_softmax, int use_provided,
+                                                   void *__restrict__ y_vals, int16_t *__restrict__ y_indx,
+                                                   int64_t y_stride, uint32_t *__restrict__ bits,
+                                                   int64_t bits_stride_row, int64_t bits_stride_word) {
+  constexpr int ROWS_PER_BLOCK = 256 / L;
+  const int sub = threadIdx.x % L;
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / L;
+  const bool live = row < n_rows;
+  const int64_t rrow = live ? row : 0;
+  const int64_t xoff = rrow * x_stride;
+  int my_idx = 0;
+  if (use_provided) {
+    if (sub < k) my_idx = y_indx[rrow * y_stride + sub];
+  } else {
+    uint64_t keys[EPL > 0 ? EPL : 1];
+    if constexpr (EPL > 0) {
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) {
+        int c = sub + j * L;
+        keys[j] = c < n_cols ? logit_key(load_as_f32<DT>(x, xoff + c), c) : 0ull;
+      }
+    }
+    uint64_t prev = ~0ull;
+    uint64_t mine = 0ull;
+    for (int pass = 0; pass < k; ++pass) {
+      uint64_t best = 0ull;
+      if constexpr (EPL > 0) {
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) {
+          uint64_t q = keys[j];
+          best = (q < prev && q > best) ? q : best;
+        }
+      } else {
+        for (int c = sub; c < n_cols; c += L) {
+          uint64_t q = logit_key(load_as_f32<DT>(x, xoff + c), c);
+          best = (q < prev && q > best) ? q : best;
+        }
+      }
+      best = group_max_u64<L>(best);
+      if (sub == pass) mine = best;
+      prev = best;
+    }
+    my_idx = (int)(0xFFFFu - (uint32_t)(mine & 0xFFFFull));
+  }
+  const bool slot = sub < k;
+  float v = slot ? load_as_f32<DT>(x, xoff + my_idx) : 0.f;
+  if (apply_softmax) {
+    float mx = group_max_f32<L>(slot ? v : -__builtin_inff());
+    float e = slot ? expf(v - mx) : 0.f;
+    float s = group_sum_f32<L>(e);
+    v = e / s;
+  }
+  if (live && slot) {
+    store_from_f32<DT>(y_vals, rrow * y_stride + sub, v);
+    if (!use_provided) y_indx[rrow * y_stride + sub] = (int16_t)my_idx;
+  }
+  const int n_words = (n_cols + 31) / 32;
+  const int base_lane = (threadIdx.x % kWave) - sub;
+  for (int w0 = 0; w0 < n_words; w0 += L) {
+    int w = w0 + sub;
+    uint32_t word = 0;
+    for (int j = 0; j < k; ++j) {
+      int ij = __shfl(my_idx, base_lane + j);
+      word |= ((ij >> 5) == w) ? (1u << (ij & 31)) : 0u;
+    }
+    if (live && w < n_words) bits[rrow * bits_stride_row + (int64_t)w * bits_stride_word] = word;
+  }
+}
+
+template <int DT>
+int launch_topk(const void *x, int64_t xs, int n_rows, int n_cols, int k, int sm, int prov, void *yv, int16_t *yi,
+                int64_t ys, uint32_t *bits, int64_t bsr, int64_t bsw, hipStream_t st) {
+  int need = (n_cols + 7) / 8;
+  if (need < k) need = k;
+#define TAMD_TOPK(LL, EE)                                                                                    \
+  topk_kernel<DT, LL, EE><<<dim3((unsigned)((n_rows + (256 / LL) - 1) / (256 / LL))), 256, 0, st>>>(          \
+      x, xs, n_rows, n_cols, k, sm, prov, yv, yi, ys, bits, bsr, bsw)
+  if (need <= 8) TAMD_TOPK(8, 8);
+  else if (need <= 16) TAMD_TOPK(16, 8);
+  else if (need <= 32) TAMD_TOPK(32, 8);
+  else if (n_cols <= 512) TAMD_TOPK(64, 8);
+  else TAMD_TOPK(64, 0);
+#undef TAMD_TOPK
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// histogram + stable expert-major ordering
+// ---------------------------------------------------------------------------
+// Entries are processed in chunks of 64 (one wave, one entry per lane).  Inside a
+// chunk the rank of an entry among the entries with the same expert is a popcount
+// of the lanes below it that hold the same id; the set of such lanes is built
+// from one ballot per bit of the id.  Per-chunk counts are prefix-summed inside a
+// block (CH chunks), per-block totals across blocks, expert totals across
+// experts; the position of an entry is the sum of those three prefixes and its
+// in-chunk rank.  No atomics, so the order is the flat (token, slot) order.
+
+TAMD_DEVICE int load_indx(const void *p, int is16, int64_t i) {
+  return is16 ? (int)((const int16_t *)p)[i] : ((const int32_t *)p)[i];
+}
+
+TAMD_DEVICE uint64_t same_id_mask(int e, bool valid, int nbits) {
+  uint64_t same = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    bool bit = (e >> b) & 1;
+    uint64_t m = __ballot(valid && bit);
+    same &= bit ? m : ~m;
+  }
+  return same;
+}
+
+TAMD_DEVICE uint64_t lanemask_lt() {
+  int lane = threadIdx.x % kWave;
+  return lane == 0 ? 0ull : (~0ull >> (64 - lane));
+}
+
+__global__ __launch_bounds__(256) void hist_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
+                                                   int CH, int nbits, int32_t *__restrict__ chunk_pref,
+                                                   int32_t *__restrict__ block_tot) {
+  extern __shared__ int32_t hist[];  // [CH][E]
+  const int blk = blockIdx.x;
+  for (int i = threadIdx.x; i < CH * E; i += 256) hist[i] = 0;
+  __syncthreads();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  for (int c = wave; c < CH; c += 4) {
+    int64_t i = ((int64_t)blk * CH + c) * 64 + lane;
+    int e = i < n ? load_indx(indx, is16, i) : -1;
+    bool valid = e >= 0 && e < E;
+    uint64_t same = same_id_mask(e, valid, nbits);
+    if (valid && (same & lanemask_lt()) == 0) hist[c * E + e] = __popcll(same);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int run = 0;
+    for (int c = 0; c < CH; ++c) {
+      int t = hist[c * E + e];
+      chunk_pref[((int64_t)blk * CH + c) * E + e] = run;
+      run += t;
+    }
+    block_tot[(int64_t)blk * E + e] = run;
+  }
+}
+
+// Exclusive scan of up to 1024 ints held one per thread; returns the total.
+TAMD_DEVICE int block_excl_scan_1024(int v, int &total, int *lds /* >= 17 ints */) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int t = __shfl_up(inc, o);
+    if (lane >= o) inc += t;
+  }
+  __syncthreads();
+  if (lane == kWave - 1) lds[wave] = inc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int w = 0; w < 16; ++w) {
+      int t = lds[w];
+      lds[w] = run;
+      run += t;
+    }
+    lds[16] = run;
+  }
+  __syncthreads();
+  total = lds[16];
+  return inc - v + lds[wave];
+}
+
+__global__ __launch_bounds__(1024) void scan_kernel(int E, int n_blocks, int32_t *__restrict__ block_tot,
+                                                    int32_t *__restrict__ col_sum, int32_t *__restrict__ col_offs,
+                                                    int32_t *__restrict__ n_valid) {
+  __shared__ int lds[17];
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 1024) {
+    int e = e0 + threadIdx.x;
+    int run = 0;
+    if (e < E) {
+#pragma unroll 4
+      for (int b = 0; b < n_blocks; ++b) {
+        int t = block_tot[(int64_t)b * E + e];
+        block_tot[(int64_t)b * E + e] = run;
+        run += t;
+      }
+      col_sum[e] = run;
+    }
+    int total;
+    int ex = block_excl_scan_1024(run, total, lds);
+    if (e < E) col_offs[e] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0) *n_valid = carry;
+}
+
+__global__ __launch_bounds__(256) void order_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
+                                                    int CH, int nbits, int k, const int32_t *__restrict__ chunk_pref,
+                                                    const int32_t *__restrict__ block_off,
+                                                    const int32_t *__restrict__ col_offs,
+                                                    const int32_t *__restrict__ n_valid,
+                                                    int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
+                                                    int32_t *__restrict__ gather) {
+  const int blk = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nv = *n_valid;
+  for (int c = wave; c < CH; c += 4) {
+    int64_t chunk = (int64_t)blk * CH + c;
+    int64_t i = chunk * 64 + lane;
+    int e = i < n ? load_indx(indx, is16, i) : -1;
+    bool valid = e >= 0 && e < E;
+    uint64_t same = same_id_mask(e, valid, nbits);
+    if (valid) {
+      int pos = col_offs[e] + block_off[(int64_t)blk * E + e] + chunk_pref[chunk * E + e] +
+                __popcll(same & lanemask_lt());
+      row_sorted[i] = pos;
+      col_sorted[pos] = (int32_t)i;
+      if (gather) gather[pos] = (int32_t)(i / k);
+    } else if (i < n) {
+      row_sorted[i] = -1;
+    }
+    if (i >= nv && i < n) {
+      col_sorted[i] = -1;
+      if (gather) gather[i] = 0;  // trunc(-1 / k)
+    }
+  }
+}
+
+struct MetaPlan {
+  int CH;
+  int nbits;
+  int64_t n_chunks, n_blocks;
+  int64_t off_chunk_pref, off_block_tot, off_col_offs, off_n_valid, total;
+};
+
+inline MetaPlan make_meta_plan(int64_t n_indx, int E) {
+  MetaPlan p;
+  // LDS histogram of CH*E ints, at most 64 KiB
+  int ch = 16;
+  while (ch > 1 && (int64_t)ch * E * 4 > 65536) ch >>= 1;
+  p.CH = ch;
+  p.nbits = 0;
+  while ((1 << p.nbits) < E) ++p.nbits;
+  p.n_chunks = (n_indx + 63) / 64;
+  p.n_blocks = (p.n_chunks + ch - 1) / ch;
+  if (p.n_blocks < 1) p.n_blocks = 1;
+  p.off_chunk_pref = 0;
+  p.off_block_tot = p.n_blocks * ch * (int64_t)E;
+  p.off_col_offs = p.off_block_tot + p.n_blocks * (int64_t)E;
+  p.off_n_valid = p.off_col_offs + E;
+  p.total = p.off_n_valid + 1;
+  return p;
+}
+
+inline int launch_bitmatrix_metadata(const void *indx, int is16, int64_t n, int E, int k, int32_t *col_sum,
+                                     int32_t *col_sorted, int32_t *row_sorted, int32_t *gather, int32_t *ws,
+                                     hipStream_t st, bool before_order(void *), void *ctx) {
+  MetaPlan p = make_meta_plan(n, E);
+  size_t lds = (size_t)p.CH * E * 4;
+  hist_kernel<<<dim3((unsigned)p.n_blocks), 256, lds, st>>>(indx, is16, n, E, p.CH, p.nbits, ws + p.off_chunk_pref,
+                                                           ws + p.off_block_tot);
+  scan_kernel<<<1, 1024, 0, st>>>(E, (int)p.n_blocks, ws + p.off_block_tot, col_sum, ws + p.off_col_offs,
+                                  ws + p.off_n_valid);
+  if (before_order && !before_order(ctx)) return launch_status();
+  order_kernel<<<dim3((unsigned)p.n_blocks), 256, 0, st>>>(indx, is16, n, E, p.CH, p.nbits, k, ws + p.off_chunk_pref,
+                                                          ws + p.off_block_tot, ws + p.off_col_offs,
+                                                          ws + p.off_n_valid, col_sorted, row_sorted, gather);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// ragged tensor metadata
+// ---------------------------------------------------------------------------
+// One block.  Wave r < 6 scans row r of the offsets table (r = 0: slice offsets,
+// r >= 1: block offsets for block size 8 << r); then all 16 waves fill the
+// schedule, one (block size, slice) pair at a time with lanes over its blocks.
+__global__ __launch_bounds__(1024) void ragged_kernel(const int32_t *__restrict__ sizes, int S,
+                                                      int32_t *__restrict__ offs, int64_t offs_pitch,
+                                                      int32_t *__restrict__ sched, int64_t sched_pitch, int max_blocks) {
+  __shared__ int totals[6];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (wave < 6) {
+    const int sh = wave == 0 ? 0 : wave + 3;
+    int32_t *row = offs + (int64_t)wave * offs_pitch;
+    int carry = 0;
+    for (int s0 = 0; s0 < S; s0 += kWave) {
+      int s = s0 + lane;
+      int v = s < S ? ((sizes[s] + ((1 << sh) - 1)) >> sh) : 0;
+      int inc = v;
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        int t = __shfl_up(inc, o);
+        if (lane >= o) inc += t;
+      }
+      if (s < S) row[s] = carry + inc - v;
+      carry += __shfl(inc, kWave - 1);
+    }
+    if (lane == 0) {
+      row[S] = carry;
+      totals[wave] = carry;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+  for (int p = wave; p < 5 * S; p += 16) {
+    const int b = p / S, s = p - b * S;
+    const int sh = b + 4;
+    const int nb = (sizes[s] + ((1 << sh) - 1)) >> sh;
+    const int start = offs[(int64_t)(b + 1) * offs_pitch + s];
+    int32_t *row = sched + (int64_t)b * sched_pitch;
+    for (int i = lane; i < nb; i += kWave) {
+      int j = start + i;
+      if (j < max_blocks) row[j] = (i << 16) + s;
+    }
+  }
+  for (int b = 0; b < 5; ++b) {
+    int32_t *row = sched + (int64_t)b * sched_pitch;
+    for (int j = totals[b + 1] + (int)threadIdx.x; j < max_blocks; j += 1024) row[j] = -1;
+  }
+}
+
+}  // namespace tamd
+
+using namespace tamd;
+
+extern "C" int tamd_topk_forward(const void *x, int x_dtype, int64_t x_stride, int n_rows, int n_cols, int k,
+                                 int apply_softmax, int use_provided_indx, void *y_vals, int16_t *y_indx,
+                                 int64_t y_stride, uint32_t *bits, int64_t bits_stride_row,
+                                 int64_t bits_stride_word, void *stream) {
+  if (n_rows < 0 || n_cols <= 0 || n_cols >= 32768 || k < 1 || k > 64 || k > n_cols) return TAMD_E_INVALID;
+  if (n_rows == 0) return 0;
+  if (!x || !y_vals || !y_indx || !bits) return TAMD_E_INVALID;
+  hipStream_t st = (hipStream_t)stream;
+  switch (x_dtype) {
+    case TAMD_F32:
+      return launch_topk<TAMD_F32>(x, x_stride, n_rows, n_cols, k, apply_softmax, use_provided_indx, y_vals, y_indx,
+                                   y_stride, bits, bits_stride_row, bits_stride_word, st);
+    case TAMD_BF16:
+      return launch_topk<TAMD_BF16>(x, x_stride, n_rows, n_cols, k, apply_softmax, use_provided_indx, y_vals, y_indx,
+                                    y_stride, bits, bits_stride_row, bits_stride_word, st);
+    case TAMD_F16:
+      return launch_topk<TAMD_F16>(x, x_stride, n_rows, n_cols, k, apply_softmax, use_provided_indx, y_vals, y_indx,
+                                   y_stride, bits, bits_stride_row, bits_stride_word, st);
+    default:
+      return TAMD_E_INVALID;
+  }
+}
+
+extern "C" int64_t tamd_bitmatrix_metadata_workspace(int64_t n_indx, int n_cols) {
+  if (n_indx < 0 || n_cols <= 0) return 0;
+  return make_meta_plan(n_indx, n_cols).total;
+}
+
+extern "C" int tamd_bitmatrix_metadata(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols,
+                                       int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                       int32_t *workspace, void *stream) {
+  if (n_indx < 0 || n_cols <= 0 || n_cols > 16384 || n_indx > 0x7FFFFFFF) return TAMD_E_INVALID;
+  if (!col_sum || !workspace || (n_indx > 0 && (!indx || !col_sorted_indx || !row_sorted_indx))) return TAMD_E_INVALID;
+  return launch_bitmatrix_metadata(indx, indx_is_int16, n_indx, n_cols, 1, col_sum, col_sorted_indx, row_sorted_indx,
+                                   nullptr, workspace, (hipStream_t)stream, nullptr, nullptr);
+}
+
+static int ragged_launch(const int32_t *slice_sizes, int n_slices, int32_t *offs, int64_t offs_pitch,
+                         int32_t *schedule, int64_t sched_pitch, int max_n_blocks, hipStream_t st) {
+  ragged_kernel<<<1, 1024, 0, st>>>(slice_sizes, n_slices, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
+  return launch_status();
+}
+
+extern "C" int tamd_ragged_metadata(const int32_t *slice_sizes, int n_slices, int32_t *offs, int64_t offs_pitch,
+                                    int32_t *schedule, int64_t sched_pitch, int max_n_blocks, void *stream) {
+  if (n_slices < 0 || n_slices > 65535 || max_n_blocks < 0 || offs_pitch < n_slices + 1 ||
+      sched_pitch < max_n_blocks)
+    return TAMD_E_INVALID;
+  if (!offs || (n_slices > 0 && !slice_sizes) || (max_n_blocks > 0 && !schedule)) return TAMD_E_INVALID;
+  return ragged_launch(slice_sizes, n_slices, offs, offs_pitch, schedule, sched_pitch, max_n_blocks,
+                       (hipStream_t)stream);
+}
+
+namespace {
+struct RaggedCtx {
+  const int32_t *sizes;
+  int n_slices;
+  int32_t *offs;
+  int64_t offs_pitch;
+  int32_t *sched;
+  int64_t sched_pitch;
+  int max_blocks;
+  hipStream_t st;
+};
+bool ragged_between(void *p) {
+  RaggedCtx *c = (RaggedCtx *)p;
+  return ragged_launch(c->sizes, c->n_slices, c->offs, c->offs_pitch, c->sched, c->sched_pitch, c->max_blocks,
+                       c->st) == 0;
+}
+}  // namespace
+
+extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
+                                     int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                     int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
+                                     int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream) {
+  if (n_indx < 0 || n_cols <= 0 || n_cols > 16384 || n_indx > 0x7FFFFFFF || k < 1) return TAMD_E_INVALID;
+  if (max_n_blocks < 0 || offs_pitch < n_cols + 1 || sched_pitch < max_n_blocks) return TAMD_E_INVALID;
+  if (!col_sum || !workspace || !offs || (max_n_blocks > 0 && !schedule)) return TAMD_E_INVALID;
+  if (n_indx > 0 && (!indx || !col_sorted_indx || !row_sorted_indx)) return TAMD_E_INVALID;
+  RaggedCtx ctx{col_sum, n_cols, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, (hipStream_t)stream};
+  return launch_bitmatrix_metadata(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx,
+                                   row_sorted_indx, gather_indx, workspace, (hipStream_t)stream, ragged_between, &ctx);
+}

@@ -1,0 +1,242 @@
+"""`matmul` (alias `matmul_ogs`): gather -> grouped / dense GEMM -> bias, fused
+activation, gamma -> scatter (matmul.py:243-749 of the reference), over the
+gfx950 kernels.  Argument names, defaults and error behaviour follow the
+reference; combinations that are not built raise NotImplementedError."""
+import ctypes
+from dataclasses import dataclass
+from typing import Callable, Optional
+
+import torch
+
+from . import _lib
+from .matmul_details import opt_flags as _opt_flags
+from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_opt_flags, scoped_opt_flags,
+                                       scoped_opt_flags_constraints)
+from .numerics import InFlexData, OutFlexData
+from .specialize import FnSpecs
+from .tensor import FP4, RaggedTensorMetadata, Tensor, wrap_torch_tensor
+
+__all__ = ["matmul", "matmul_ogs", "PrecisionConfig", "FlexCtx", "FusedActivation", "Epilogue", "FnSpecs",
+           "InFlexData", "OutFlexData", "InapplicableConstraint", "OptFlags", "scoped_opt_flags",
+           "scoped_opt_flags_constraints"]
+
+MXFP_BLOCK_SIZE = 32
+
+
+@dataclass(frozen=True)
+class FusedActivation:
+    specs: FnSpecs = FnSpecs.default()
+    fn_args: tuple = tuple()
+
+
+@dataclass(frozen=True)
+class Epilogue:
+    specs: FnSpecs = FnSpecs.default()
+    fn_arg_values_matmul: tuple = tuple()
+    fn_arg_values_finalize: tuple = tuple()
+    effective_itemsize: Optional[float] = None
+
+
+@dataclass(frozen=True)
+class FlexCtx:
+    lhs_data: InFlexData = InFlexData()
+    rhs_data: InFlexData = InFlexData()
+    out_data: OutFlexData = OutFlexData()
+    acc_data: InFlexData = InFlexData()
+
+
+@dataclass
+class PrecisionConfig:
+    max_num_imprecise_acc: Optional[int] = None
+    allow_tf32: bool = True
+    flex_ctx: FlexCtx = FlexCtx()
+    acc_scale: float = 1.0
+    flexpoint_saturate_inf: bool = False
+    report_quantization_err_fn: Optional[Callable] = None
+    a_mx_scale: Optional[torch.Tensor] = None
+    a_mx_tensor_scale: Optional[torch.Tensor] = None
+    a_microblock_size: Optional[int] = None
+    b_mx_scale: Optional[torch.Tensor] = None
+    b_mx_tensor_scale: Optional[torch.Tensor] = None
+    b_microblock_size: Optional[int] = None
+    c_mx_scale: Optional[torch.Tensor] = None
+    c_microblock_size: Optional[int] = None
+    c_value_pack_factor: int = 1
+    out_dtype: Optional[torch.dtype] = None
+    intermediate_out_dtype: Optional[torch.dtype] = None
+    enforce_bitwise_invariance: bool = False
+
+
+def _data(t):
+    return t.storage.data if isinstance(t, Tensor) else t
+
+
+def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
+           b_ragged_metadata: Optional[RaggedTensorMetadata] = None, gather_indx: Optional[torch.Tensor] = None,
+           scatter_indx: Optional[torch.Tensor] = None, precision_config: Optional[PrecisionConfig] = None,
+           betas: Optional[torch.Tensor] = None, gammas: Optional[torch.Tensor] = None,
+           out_alpha: Optional[float] = None, c: Optional[torch.Tensor] = None, fused_comm=None,
+           fused_activation: Optional[FusedActivation] = None, epilogue: Optional[Epilogue] = None,
+           c_acc_in: Optional[torch.Tensor] = None):
+    """
+    Y[dst(r), :] = act((X[src(r), :] @ W[e]) + bias[e] * betas[r]) * gammas[r]   for the rows r of every slice e
+
+    a: [M, K] activations (bf16 / fp16), or [B, M, K] batched.
+    b: [E, K, N] weights; MXFP4 weights are uint8 with two codes per byte along K
+       (storage [E, K/2, N] with unit stride along K) and precision_config.b_mx_scale
+       holds their e8m0 scales [E, K/32, N].
+    a_ragged_metadata: rows of `a` (after gather) are grouped by slice.
+    gather_indx / scatter_indx: int32 row maps (scatter -1 drops the row).
+    """
+    if precision_config is None:
+        precision_config = PrecisionConfig()
+    if fused_activation is None:
+        fused_activation = FusedActivation(FnSpecs.default(), tuple())
+    if epilogue is None:
+        epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+    is_input_batched = a.ndim == 3
+    if is_input_batched:
+        assert gather_indx is None, "gather not supported in batched mode"
+        assert scatter_indx is None, "scatter not supported in batched mode"
+        assert b_ragged_metadata is None, "w cannot be ragged in batched mode"
+        assert a_ragged_metadata is None, "x cannot be ragged in batched mode"
+        assert fused_comm is None, "fused comm is not supported in batched mode"
+        assert b.ndim == 3 and b.shape[0] == a.shape[0]
+    if b_ragged_metadata is not None:
+        raise NotImplementedError("K-ragged matmul is not built for gfx950")
+    if fused_comm is not None:
+        raise NotImplementedError("fused communication needs more than one GPU")
+    if c_acc_in is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
+        raise NotImplementedError("accumulator input / quantising epilogues are not built")
+    if precision_config.a_mx_scale is not None:
+        raise NotImplementedError("microscaled activations are not built")
+    flex = precision_config.flex_ctx
+    if flex.out_data.expected_scale is not None or flex.out_data.actual_scale is not None \
+            or flex.acc_data.scale is not None:
+        raise NotImplementedError("flexpoint output scaling is not built")
+    # ---- weights
+    b_scale = precision_config.b_mx_scale
+    if not isinstance(b, Tensor):
+        b = wrap_torch_tensor(b, dtype=FP4 if b.dtype == torch.uint8 else None)
+    if b_scale is not None:
+        assert precision_config.b_microblock_size is not None, \
+            "precision_config.b_microblock_size is required when precision_config.b_mx_scale is set"
+        assert precision_config.b_microblock_size == MXFP_BLOCK_SIZE, "Unsupported microscale block size"
+        b_scale = _data(b_scale)
+        assert b_scale.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.dtype}"
+    if isinstance(a, Tensor):
+        a = a.storage.data
+    a = flex.lhs_data.reinterpret(a)
+    w = flex.rhs_data.reinterpret(b.storage.data)
+    _lib.require_gpu(a, "a")
+    _lib.require_gpu(w, "b")
+    assert a.stride(-1) == 1 or a.shape[-1] == 1, "a must be contiguous along K"
+    # ---- shapes
+    K = a.shape[-1]
+    K_W, N = b.shape[-2:]
+    assert K == K_W, f"inner dimensions differ: {K} vs {K_W}"
+    ragged = a_ragged_metadata is not None
+    M = a.shape[-2] if gather_indx is None else gather_indx.shape[0]
+    if ragged:
+        n_slices, batch = a_ragged_metadata.n_slices, 1
+    elif b.ndim == 3:
+        n_slices = batch = b.shape[0]
+    else:
+        n_slices = batch = 1
+    red_n = fused_activation.specs.reduction_n
+    out_dtype = precision_config.out_dtype or a.dtype
+    rows_out = M
+    if gather_indx is not None:
+        rows_out = gather_indx.shape[0]
+    if scatter_indx is not None:
+        rows_out = scatter_indx.shape[0]
+    out_shape = (batch, rows_out, N // red_n)
+    if c is None:
+        out = torch.empty(out_shape, dtype=out_dtype, device=a.device)
+    else:
+        out = c[None] if c.ndim == 2 else c
+        assert tuple(out.shape) == out_shape, f"output shape {tuple(out.shape)} != {out_shape}"
+        assert out.stride(-1) == 1
+    squeeze = not is_input_batched
+
+    def finish():
+        return out.squeeze(0) if squeeze else out
+
+    if batch * M * N == 0:
+        return finish()
+    # ---- activation
+    act, act_alpha, act_limit, has_limit = _lib.ACT_NONE, 0.0, 0.0, 0
+    if fused_activation.specs.name == "swiglu":
+        assert red_n == 2
+        named = dict(zip(fused_activation.specs.fn_arg_names, fused_activation.fn_args))
+        act = _lib.ACT_SWIGLU
+        act_alpha = float(named.get("alpha", fused_activation.fn_args[0]))
+        limit = named.get("limit", fused_activation.fn_args[1] if len(fused_activation.fn_args) > 1 else None)
+        has_limit = int(limit is not None)
+        act_limit = float(limit) if limit is not None else 0.0
+    elif fused_activation.specs.name != "dflt":
+        raise NotImplementedError(f"fused activation {fused_activation.specs.name!r} is not built")
+    # ---- tile choice
+    flags = make_opt_flags(M, N, K, n_slices, ragged,
+                           a_ragged_metadata.expected_slice_size if ragged else None)
+    args = _lib.MatmulArgs()
+    args.x, args.x_dtype = a.data_ptr(), _lib.dtype_code(a.dtype)
+    args.x_stride_m = a.stride(-2)
+    args.x_stride_z = a.stride(0) if a.ndim == 3 else 0
+    args.x_scale = None if flex.lhs_data.scale is None else flex.lhs_data.scale.data_ptr()
+    wd = w if w.ndim == 3 else w[None]
+    args.w = wd.data_ptr()
+    if b.dtype == FP4:
+        assert b_scale is not None, "MXFP4 weights need precision_config.b_mx_scale"
+        args.w_dtype = _lib.MXFP4
+        sd = b_scale if b_scale.ndim == 3 else b_scale[None]
+        assert tuple(sd.shape) == (wd.shape[0], K // MXFP_BLOCK_SIZE, N), \
+            f"b_mx_scale shape {tuple(sd.shape)} != {(wd.shape[0], K // MXFP_BLOCK_SIZE, N)}"
+        args.w_mx_scale = sd.data_ptr()
+        args.w_mx_stride_e, args.w_mx_stride_k, args.w_mx_stride_n = sd.stride()
+    else:
+        args.w_dtype = _lib.dtype_code(w.dtype)
+    args.w_stride_e, args.w_stride_k, args.w_stride_n = wd.stride()
+    args.w_scale = None if flex.rhs_data.scale is None else flex.rhs_data.scale.data_ptr()
+    if bias is not None:
+        bb = bias if bias.ndim == 2 else bias[None]
+        assert bb.stride(-1) == 1 and bb.shape[-1] == N
+        args.bias, args.bias_dtype, args.bias_stride_e = bb.data_ptr(), _lib.dtype_code(bb.dtype), bb.stride(0)
+    keep = []  # temporaries that must outlive the launch call
+
+    def f32(t):
+        if t is None:
+            return None
+        t = t if t.dtype == torch.float32 and t.is_contiguous() else t.to(torch.float32).contiguous()
+        keep.append(t)
+        return t.data_ptr()
+
+    def i32(t):
+        if t is None:
+            return None
+        t = t if t.dtype == torch.int32 and t.is_contiguous() else t.to(torch.int32).contiguous()
+        keep.append(t)
+        return t.data_ptr()
+
+    args.betas, args.gammas = f32(betas), f32(gammas)
+    args.out_alpha = 1.0 if out_alpha is None else float(out_alpha)
+    args.y, args.y_dtype = out.data_ptr(), _lib.dtype_code(out.dtype)
+    args.y_stride_m, args.y_stride_z = out.stride(1), out.stride(0)
+    args.M, args.N, args.K, args.n_experts = M, N, K, n_slices
+    args.gather_indx, args.scatter_indx = i32(gather_indx), i32(scatter_indx)
+    if ragged:
+        md = a_ragged_metadata
+        args.slice_sizes, args.slice_offs = md.slice_sizes.data_ptr(), md.slice_offs.data_ptr()
+        args.block_offs = md.block_offs(flags.block_m).data_ptr()
+        args.block_schedule = md.block_schedule(flags.block_m).data_ptr()
+        args.block_m = flags.block_m
+        args.grid_m = RaggedTensorMetadata.n_blocks(md.n_slices, M, flags.block_m)
+    else:
+        args.force_variant = flags.block_m if "block_m" in _opt_flags._constraints() else 0
+    args.activation, args.act_alpha, args.act_limit, args.act_has_limit = act, act_alpha, act_limit, has_limit
+    rc = _lib.lib().tamd_matmul(ctypes.byref(args), _lib.stream_ptr(a.device))
+    _lib.check(rc, "matmul")
+    return finish()
+
+
+matmul_ogs = matmul
