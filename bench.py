@@ -1,0 +1,190 @@
+"""Benchmark of the quantized-MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload fc1_prefill|fc1_decode|dense|routing]
+
+Default workload: MoE up-projection + fused SwiGLU at the prefill shape (T=4096 tokens, hidden 2880,
+128 experts, top-4, MXFP4 weights [128, 2880, 5760], bf16 activations).  A step is one pass of the path over
+one batch: routing(logits) then matmul_ogs(gather -> grouped GEMM -> bias + SwiGLU).  Inputs (logits,
+activations, quantised weights) are resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_MXFP4_TFLOPS = 10100.0
+
+WORKLOADS = {
+    # name: (T, E, k, K, N, swiglu)
+    "fc1_prefill": dict(T=4096, E=128, k=4, K=2880, N=5760, act=True),
+    "fc1_decode": dict(T=64, E=128, k=4, K=2880, N=5760, act=True),
+}
+
+
+def make_weights(E, K, N, device, seed=0):
+    """W ~ N(0, 0.02) fp32 generated and quantised to MXFP4 along K one expert at a time."""
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+    from triton_amd.tensor import FP4, empty
+    from triton_amd.tensor_details.dtype import UINT8
+    from triton_amd.tensor_details.layout import StridedLayout
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    vals = empty((E, K, N), FP4, device, StridedLayout(-2)).storage.data
+    scales = empty((E, K // 32, N), UINT8, device, StridedLayout(-2)).storage.data
+    for e in range(E):
+        w = torch.randn((1, K, N), generator=g, device=device, dtype=torch.float32) * 0.02
+        v, s = downcast_to_mxfp(w, torch.uint8, axis=1)
+        vals[e].copy_(v[0])
+        scales[e].copy_(s[0])
+    return vals, scales
+
+
+def algorithmic_bytes(col_sum, T, k, K, N, act):
+    """x rows read + y rows written + (codes + scales + bias) of the experts that have rows."""
+    rows = T * k
+    n_active = int((col_sum > 0).sum())
+    n_out = N // 2 if act else N
+    per_expert = K // 2 * N + K // 32 * N + N * 2
+    return rows * K * 2 + rows * n_out * 2 + n_active * per_expert, n_active
+
+
+def cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, experts, K, N, act):
+    """Oracle (CPU restatement of the reference's torch path) timed on a bounded sample: the first
+    `experts` experts of the same workload, all host cores."""
+    from oracle import matmul_ref as MR
+    torch.set_num_threads(os.cpu_count())
+    sizes = ref["col_sum"][:experts]
+    n_rows = int(sizes.sum())
+    gather = ref["gather_indx"][:n_rows]
+    v = vals[:experts].cpu()
+    s = scales[:experts].cpu()
+    t0 = time.perf_counter()
+    y = MR.matmul_ref(x_cpu, v, bias_cpu[:experts], slice_sizes=sizes, gather_indx=gather, b_mx_scale=s,
+                      fused_swiglu=(1.702, 7.0) if act else None)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * n_rows * K * N
+    return y, n_rows, flops / dt / 1e12, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fc1_prefill", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-experts", type=int, default=8, help="experts in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--block-m", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (experts would shard across GPUs, "
+              "see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+
+    from oracle import routing_ref as RR
+    from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
+    from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
+    from triton_amd.routing import routing
+    from triton_amd.swiglu import swiglu_fn
+
+    cfg = WORKLOADS[args.workload]
+    T, E, k, K, N, act = cfg["T"], cfg["E"], cfg["k"], cfg["K"], cfg["N"], cfg["act"]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    logits_cpu = torch.randn(T, E)
+    x_cpu = torch.randn(T, K).to(torch.bfloat16)
+    bias_cpu = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
+    logits, x, bias = logits_cpu.to(dev), x_cpu.to(dev), bias_cpu.to(dev)
+    vals, scales = make_weights(E, K, N, dev)
+    pc = PrecisionConfig(b_mx_scale=scales, b_microblock_size=32)
+    fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if act else None
+    constraints = {"block_m": args.block_m} if args.block_m else {}
+
+    def step(ev=None):
+        r = routing(logits, k)
+        if ev is not None:
+            ev[0].record()
+        y = matmul(x, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=fa)
+        if ev is not None:
+            ev[1].record()
+        return r, y
+
+    with scoped_opt_flags_constraints(constraints):
+        for _ in range(args.warmup):
+            r, y = step()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        for i in range(args.steps):
+            r, y = step(events[i])
+        stop.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+
+    col_sum = r.col_sum.cpu()
+    rows = T * k
+    flops = 2.0 * rows * K * N
+    abytes, n_active = algorithmic_bytes(col_sum, T, k, K, N, act)
+    tflops_step = flops / (ms_per_step * 1e-3) / 1e12
+    tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
+    gbs_kernel = abytes / (kernel_ms * 1e-3) / 1e9
+    hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (PEAK_BF16_TFLOPS * 1e12))
+    if hbm_bound:
+        roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=None)
+    else:
+        roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                    frac=round(tflops_kernel / PEAK_BF16_TFLOPS, 4), traffic=None)
+    roof["kernel"] = "mm_x16_mxfp4_kernel"
+    roof["kernel_ms"] = round(kernel_ms, 4)
+    roof["algorithmic_bytes"] = abytes
+    roof["algorithmic_flops"] = flops
+    roof["frac_of_mxfp4_peak"] = round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4)
+    roof["hbm_gbs"] = round(gbs_kernel, 1)
+
+    # parity of this very run against the oracle, and the CPU baseline, on a bounded sample
+    ref = RR.routing_ref(logits_cpu, k)
+    routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(col_sum, ref["col_sum"])
+                      and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]))
+    cpu = None
+    gemm_ok = None
+    if args.cpu_experts > 0:
+        n_e = min(args.cpu_experts, E)
+        y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, n_e, K, N, act)
+        gemm_ok = bool(torch.allclose(y[:n_rows].cpu().float(), y_ref.float(), rtol=1e-2, atol=1e-2))
+        cpu = dict(value=round(cpu_tflops, 5), unit="TFLOP/s", cores=os.cpu_count(), kind="port",
+                   sample=f"oracle matmul_ref (dequantise + fp32 GEMM + SwiGLU) on the first {n_e} of {E} experts "
+                          f"({n_rows} of {rows} rows), {cpu_s:.1f} s")
+    out = {
+        "metric": "moe_matmul_ogs_tflops", "value": round(tflops_step, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x mxfp4 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: routing + matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, "
+                               f"hidden={K}, experts={E}, top-{k}, W1 mxfp4 [{E},{K},{N}]",
+                   "rows": rows, "active_experts": n_active},
+        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
+        "matmul_kernel_tflops": round(tflops_kernel, 2),
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "parity": {"routing_bit_exact": routing_ok, "gemm_sample_within_1e-2": gemm_ok},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
