@@ -26,6 +26,8 @@ WORKLOADS = {
     # name: (T, E, k, K, N, swiglu)
     "fc1_prefill": dict(T=4096, E=128, k=4, K=2880, N=5760, act=True),
     "fc1_decode": dict(T=64, E=128, k=4, K=2880, N=5760, act=True),
+    # same rows and FLOPs as fc1_prefill with few experts: weights (66 MB) stay cache resident
+    "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
 }
 
 

@@ -197,6 +197,8 @@ typedef struct tamd_matmul_args {
   int act_has_limit;
   /* tuning overrides (0 = heuristic) */
   int force_variant;
+  /* rows of x addressable through gather_indx (0 = M); x_rows * x_stride_m must stay below 2^30 elements */
+  int64_t x_rows;
 } tamd_matmul_args;
 
 int tamd_matmul(const tamd_matmul_args *args, void *stream);

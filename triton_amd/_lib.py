@@ -48,7 +48,7 @@ class MatmulArgs(C.Structure):
         ("block_m", C.c_int), ("grid_m", C.c_int),
         ("x_stride_z", C.c_int64), ("y_stride_z", C.c_int64),
         ("activation", C.c_int), ("act_alpha", C.c_float), ("act_limit", C.c_float), ("act_has_limit", C.c_int),
-        ("force_variant", C.c_int),
+        ("force_variant", C.c_int), ("x_rows", C.c_int64),
     ]
 
 

@@ -5,19 +5,24 @@
 // (matmul_details/_matmul.py:43-669 of the reference; epilogue order :540-559.)
 //
 // Work decomposition
-//   workgroup (4 waves) = one BLOCK_M x BLOCK_N output tile of one expert, taken from
-//     the ragged block schedule ((block << 16) | expert, -1 = padding);
-//   wave w owns the 16*NF columns [w*16*NF, (w+1)*16*NF) of the tile and ALL its rows:
-//     the MXFP4 weights of those columns go HBM -> registers (one 128-bit load = 32
-//     consecutive K of one column = one e8m0 group), are expanded to bf16/f16 in
-//     registers with v_cvt_scalef32_pk_*_fp4 and feed v_mfma_f32_16x16x32 as the B
-//     operand, so every weight byte is fetched and converted once per workgroup;
-//   the activation rows (gathered) are staged through LDS, double buffered, 128 K
-//     per stage, 16-byte chunks XOR-swizzled by row so that the MFMA A-operand reads
-//     (16 rows x one chunk per quarter-wave) hit distinct banks.
+//   workgroup (4 waves) = one BLOCK_M x 256 output tile of one expert, taken from the ragged
+//     block schedule ((block << 16) | expert, -1 = padding);
+//   wave w owns the 64 columns [64w, 64w+64) of the tile and ALL its rows: the MXFP4 weights
+//     of those columns go HBM -> registers (one 128-bit load = 32 consecutive K of one column =
+//     one e8m0 group), are expanded to bf16/f16 in registers with v_cvt_scalef32_pk_*_fp4 and
+//     feed v_mfma_f32_32x32x16 as the B operand, so every weight byte is fetched and converted
+//     once per workgroup and never touches LDS;
+//   the activation rows (gathered) are staged through LDS, double buffered, 128 K per stage,
+//     16-byte chunks XOR-swizzled by row so that the MFMA A-operand reads hit distinct banks.
 //
-// K order inside a 128-K stage: lane group g = lane/16 holds K [32g, 32g+32) of its
-// column; MFMA step s consumes elements [8s, 8s+8) of every group, for A and B alike.
+// The 32x32x16 MFMA is used because it sustains twice the rate of 16x16x32 on this part
+// (measured 2.45 vs 1.25 PFLOP/s for bf16).
+//
+// K order inside a 128-K stage: lane half h = lane/32 holds K [64q + 32h, 64q + 32h + 32) of its
+// column for q = 0, 1 (two 128-bit loads); MFMA step s = 4q + u consumes elements [8u, 8u+8) of
+// load q in both halves, for A and B alike.
+#include <type_traits>
+
 #include "common.h"
 
 namespace tamd {
@@ -26,10 +31,12 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int KB = 128;            // K per pipeline stage
 constexpr int ROW_BYTES = KB * 2;  // LDS bytes per activation row per stage
+constexpr int NF = 2;              // 32-column fragments per wave
+constexpr int BLOCK_N = 4 * 32 * NF;
 
 template <int XDT>
 struct Mma;
@@ -43,8 +50,8 @@ struct Mma<TAMD_BF16> {
     bf16x2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 3);
     return frag_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
   }
-  static TAMD_DEVICE f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  static TAMD_DEVICE f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <>
@@ -57,8 +64,8 @@ struct Mma<TAMD_F16> {
     f16x2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, scale, 3);
     return frag_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
   }
-  static TAMD_DEVICE f32x4_t mma(frag_t a, frag_t b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  static TAMD_DEVICE f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -74,31 +81,32 @@ TAMD_DEVICE void store_any(void *p, int dt, int64_t i, float v) {
   else ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v);
 }
 
-TAMD_DEVICE float swiglu_epi(float g, float l, float alpha, float limit, bool has_limit) {
+// Gate for the fused epilogue (swiglu_details/_swiglu.py:55-65): exp and reciprocal on the
+// hardware transcendental unit (relative error ~1e-6, far inside the 16-bit output rounding).
+TAMD_DEVICE float swiglu_fast(float g, float l, float alpha, float limit, bool has_limit) {
   if (has_limit) {
     g = __builtin_fminf(g, limit);
     l = __builtin_fminf(__builtin_fmaxf(l, -limit), limit);
   }
-  float s = g / (1.0f + expf(-alpha * g));
+  float e = __builtin_amdgcn_exp2f(-alpha * 1.4426950408889634f * g);
+  float s = g * __builtin_amdgcn_rcpf(1.0f + e);
   return __builtin_fmaf(s, l, s);
 }
 
 // Tile coordinates of a workgroup.
 struct Tile {
-  int expert;     // weight slice
-  int z;          // batch index (dense batched) else 0
-  int start_m;    // first expert-sorted row of the slice
-  int off_m;      // first row of the tile inside the slice
-  int rows;       // valid rows in the tile (1..BLOCK_M)
-  int slice_rows; // rows of the slice
-  int n0;         // first column of the tile
+  int expert;   // weight slice
+  int z;        // batch index (dense batched) else 0
+  int start_m;  // first expert-sorted row of the slice
+  int off_m;    // first row of the tile inside the slice
+  int rows;     // valid rows in the tile (1..BLOCK_M)
+  int n0;       // first column of the tile
 };
 
-template <int BLOCK_M, int BLOCK_N>
+template <int BLOCK_M>
 TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid_total, Tile &t) {
-  // XCD-aware remap: hardware deals workgroups round-robin to the 8 XCDs; give each
-  // XCD a contiguous range of tiles so neighbours (same expert, adjacent columns)
-  // share one L2.
+  // XCD-aware remap: hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
+  // contiguous range of tiles so neighbours (same expert, adjacent columns) share one L2.
   const int64_t per_xcd = (grid_total + 7) / 8;
   int64_t pid = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (pid >= grid_total) return false;
@@ -106,12 +114,13 @@ TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid
   int pid_n = (int)(pid - (int64_t)pid_m * grid_n);
   t.n0 = pid_n * BLOCK_N;
   t.z = 0;
+  int slice_rows;
   if (a.block_schedule) {
     int sched = a.block_schedule[pid_m];
     if (sched == -1) return false;
     t.expert = sched & 0xFFFF;
     int blk = sched >> 16;
-    t.slice_rows = a.slice_sizes[t.expert];
+    slice_rows = a.slice_sizes[t.expert];
     t.start_m = a.slice_offs[t.expert];
     t.off_m = blk * BLOCK_M;
   } else {
@@ -119,140 +128,188 @@ TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid
     int z = pid_m / bm;
     t.expert = z;
     t.z = z;
-    t.slice_rows = a.M;
+    slice_rows = a.M;
     t.start_m = 0;
     t.off_m = (pid_m - z * bm) * BLOCK_M;
   }
-  t.rows = t.slice_rows - t.off_m;
+  t.rows = slice_rows - t.off_m;
   if (t.rows > BLOCK_M) t.rows = BLOCK_M;
   return t.rows > 0;
 }
 
-// MF: 16-row fragments per tile (BLOCK_M = 16*MF); NF: 16-column fragments per wave.
-template <int XDT, int MF, int NF, int ACT>
-__global__ __launch_bounds__(256) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+// 128-bit global -> LDS copy that bypasses registers (buffer_load ... lds).  The LDS destination of
+// lane L is lds_addr + 16*L; out-of-range offsets (>= num_records of the descriptor) deliver zeros.
+// Issued through inline asm so that the compiler does not serialise later LDS reads behind it; the
+// kernel waits for these copies itself (wait_dma) before the barrier that publishes a stage.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+TAMD_DEVICE void dma16(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+TAMD_DEVICE void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
+  uint64_t p = (uint64_t)base;
+  return v4i_t{__builtin_amdgcn_readfirstlane((int)(uint32_t)p),
+               __builtin_amdgcn_readfirstlane((int)((uint32_t)(p >> 32) & 0xFFFFu)), (int)num_records, 0x00020000};
+}
+
+constexpr int B_STAGE_BYTES = 4 * 64 * 64;  // 256 columns x 64 bytes (128 K of fp4) per stage
+
+// One output tile with NFR (compile time) active 32-row fragments.  LDS: NSTAGE stages of
+// [A: LDS_ROWS x 256 B | B: 4 waves x 64 columns x 64 B], then the tile's e8m0 scales.
+//
+// Both operands reach LDS by DMA, one stage ahead of the multiply.  Activations: thread (row
+// tid/16, slot tid%16) of every 16-row group fetches the 16-byte chunk slot^(row%16), so chunk c of
+// row r sits at slot c^(r%16) and the 32-row MFMA operand reads are bank-conflict free.  Weights:
+// each wave copies its own 64 columns, 64 contiguous bytes per column per stage (4 lanes x 16 B),
+// into position p' = f*32 + c (global column 2c + f of the wave's strip, so that a lane ends up
+// with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3 against conflicts.
+template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS>
+TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
-  constexpr int BLOCK_M = 16 * MF;
-  constexpr int BLOCK_N = 64 * NF;
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2][BLOCK_M * ROW_BYTES];
-
-  Tile t;
-  if (!locate_tile<BLOCK_M, BLOCK_N>(a, grid_n, grid_total, t)) return;
+  constexpr int NG = 2 * NFR;  // 16-row groups staged per K stage
+  constexpr int STAGE_BYTES = LDS_ROWS * ROW_BYTES + B_STAGE_BYTES;
+  constexpr uint32_t kOob = 0x7FFFFFFFu;
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
-  const int cidx = lane % 16, g = lane / 16;
-  const int nfr = (t.rows + 15) / 16;  // active row fragments (wave uniform)
-  const int K = a.K, N = a.N;
+  const int c32 = lane % 32, h = lane / 32;
+  const int K = a.K, N = a.N, G = K / 32;
 
-  // ---- activation staging: thread -> (row tid/16 of every fragment, chunk tid%16)
-  const int a_chunk = tid % 16, a_row = tid / 16;
-  const uint8_t *a_ptr[MF];
+  const v4i_t rx = make_rsrc((const uint8_t *)a.x + (int64_t)t.z * a.x_stride_z * 2, kOob);
+  const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
+  const uint8_t *s_base = a.w_mx_scale + (int64_t)t.expert * a.w_mx_stride_e;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  uint8_t *lds_sc = lds + 2 * STAGE_BYTES;
+
+  // ---- scales of the whole tile, once: 256 columns x G bytes, contiguous in memory
+  const int tile_cols = N - t.n0 < BLOCK_N ? N - t.n0 : BLOCK_N;
+  if constexpr (SC_LDS) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(s_base + (int64_t)t.n0 * G), 0, (uint32_t)(tile_cols * G), 0x00020000);
+    const int n_dw = (BLOCK_N * G + 3) / 4;
+    for (int i = tid; i < n_dw; i += 256)
+      ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
+  }
+
+  // ---- activation DMA: wave w copies rows 4w..4w+3 of every 16-row group
+  const int a_slot = lane % 16, a_row = wave * 4 + lane / 16;  // row inside a 16-row group
+  const int a_chunk = a_slot ^ a_row;
+  uint32_t a_off[NG];
 #pragma unroll
-  for (int i = 0; i < MF; ++i) {
+  for (int i = 0; i < NG; ++i) {
     int r = i * 16 + a_row;
     int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
-    int64_t src = a.gather_indx ? (int64_t)a.gather_indx[t.start_m + rr] : (int64_t)(t.start_m + rr);
-    a_ptr[i] = (const uint8_t *)a.x + ((int64_t)t.z * a.x_stride_z + src * a.x_stride_m) * 2 + a_chunk * 16;
+    uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
+    a_off[i] = src * (uint32_t)(a.x_stride_m * 2) + a_chunk * 16;
   }
-  // ---- weight columns of this lane
-  const uint8_t *w_ptr[NF];
-  const uint8_t *s_ptr[NF];
-  int col[NF];
+  // ---- weight DMA: instruction j copies LDS positions j*16 + lane/4, part slot lane%4
+  uint32_t w_off[4];
+  int w_part[4];
 #pragma unroll
-  for (int f = 0; f < NF; ++f) {
-    col[f] = t.n0 + wave * (16 * NF) + cidx * NF + f;
-    int cc = col[f] < N ? col[f] : N - 1;
-    w_ptr[f] = (const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e + (int64_t)cc * a.w_stride_n + g * 16;
-    s_ptr[f] = a.w_mx_scale + (int64_t)t.expert * a.w_mx_stride_e + (int64_t)cc * a.w_mx_stride_n + g;
+  for (int j = 0; j < 4; ++j) {
+    const int pos = j * 16 + lane / 4;  // f*32 + c
+    const int col = t.n0 + wave * 64 + 2 * (pos % 32) + pos / 32;
+    w_part[j] = (lane % 4) ^ ((pos >> 2) & 3);
+    w_off[j] = (uint32_t)(col < N ? col : N - 1) * (uint32_t)a.w_stride_n + w_part[j] * 16;
   }
+  // ---- this lane's MFMA columns
+  const int col0 = t.n0 + wave * 64 + c32 * NF;
 
-  f32x4_t acc[MF][NF];
+  f32x16_t acc[NFR][NF];
 #pragma unroll
-  for (int i = 0; i < MF; ++i)
+  for (int i = 0; i < NFR; ++i)
 #pragma unroll
-    for (int f = 0; f < NF; ++f) acc[i][f] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[i][f][j] = 0.f;
 
-  uint4 a_stage[MF];
-  uint4 b_raw[NF];
-  uint32_t b_scale[NF];
-
-  auto fetch = [&](int kb) {
-    const bool a_ok = kb + a_chunk * 8 < K;
+  const int n_kb = (K + KB - 1) / KB;
+  auto issue = [&](int it) {
+    const int kb = it * KB;
+    const uint32_t sb = lds_base + (it & 1) * STAGE_BYTES;
+    const uint32_t akill = kb + a_chunk * 8 < K ? 0u : kOob;
 #pragma unroll
-    for (int i = 0; i < MF; ++i) {
-      if (i < nfr) a_stage[i] = a_ok ? *(const uint4 *)(a_ptr[i] + (int64_t)kb * 2) : make_uint4(0, 0, 0, 0);
-    }
-    const bool b_ok = kb + g * 32 < K;
+    for (int i = 0; i < NG; ++i) dma16(rx, sb + (i * 16 + wave * 4) * ROW_BYTES, a_off[i] | akill, kb * 2);
+    const uint32_t bb = sb + LDS_ROWS * ROW_BYTES + wave * 4096;
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      b_raw[f] = b_ok ? *(const uint4 *)(w_ptr[f] + (kb >> 1)) : make_uint4(0, 0, 0, 0);
-      b_scale[f] = b_ok ? (uint32_t)s_ptr[f][kb >> 5] : 0u;
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t bkill = kb + w_part[j] * 32 < K ? 0u : kOob;
+      dma16(rw, bb + j * 1024, w_off[j] | bkill, kb >> 1);
     }
   };
 
-  const int n_kb = (K + KB - 1) / KB;
-  fetch(0);
-  for (int it = 0; it < n_kb; ++it) {
-    uint8_t *buf = lds[it & 1];
+  auto compute = [&](int it) {
+    const uint8_t *buf = lds + (it & 1) * STAGE_BYTES;
+    const uint8_t *bbuf = buf + LDS_ROWS * ROW_BYTES + wave * 4096;
+    uint4 raw[NF][2];
+    float scf[NF][2];
 #pragma unroll
-    for (int i = 0; i < MF; ++i) {
-      if (i < nfr) {
-        int r = i * 16 + a_row;
-        *(uint4 *)(buf + r * ROW_BYTES + ((a_chunk ^ (r & 15)) * 16)) = a_stage[i];
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int pos = f * 32 + c32;
+        raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * h + q) ^ ((pos >> 2) & 3)) * 16));
+        const int kg = it * 4 + 2 * h + q;
+        uint32_t sbyte;
+        if constexpr (SC_LDS) sbyte = lds_sc[(wave * 64 + c32 * NF + f) * G + (kg < G ? kg : G - 1)];
+        else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + (kg < G ? kg : G - 1)];
+        scf[f][q] = bits_to_f32(sbyte << 23);
       }
-    }
-    uint4 b_cur[NF];
-    float sc_cur[NF];
+    auto read_frags = [&](int s, frag_t *af) {
+      const int chunk = h * 8 + (s >> 2) * 4 + (s & 3);
 #pragma unroll
-    for (int f = 0; f < NF; ++f) {
-      b_cur[f] = b_raw[f];
-      sc_cur[f] = bits_to_f32(b_scale[f] << 23);
-    }
-    __syncthreads();
-    if (it + 1 < n_kb) fetch((it + 1) * KB);
+      for (int i = 0; i < NFR; ++i)
+        af[i] = *(const frag_t *)(buf + (i * 32 + c32) * ROW_BYTES + ((chunk ^ (c32 & 15)) * 16));
+    };
+    frag_t af[2][NFR];
+    read_frags(0, af[0]);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      frag_t af[MF];
-#pragma unroll
-      for (int i = 0; i < MF; ++i) {
-        if (i < nfr) {
-          int r = i * 16 + cidx;
-          af[i] = *(const frag_t *)(buf + r * ROW_BYTES + (((g * 4 + s) ^ (r & 15)) * 16));
-        }
-      }
+    for (int s = 0; s < 8; ++s) {
+      if (s < 7) read_frags(s + 1, af[(s + 1) & 1]);
+      const int q = s >> 2, u = s & 3;
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
-        uint32_t codes = s == 0 ? b_cur[f].x : (s == 1 ? b_cur[f].y : (s == 2 ? b_cur[f].z : b_cur[f].w));
-        frag_t bf = M::expand(codes, sc_cur[f]);
+        const uint4 r = raw[f][q];
+        const uint32_t codes = u == 0 ? r.x : (u == 1 ? r.y : (u == 2 ? r.z : r.w));
+        const frag_t bf = M::expand(codes, scf[f][q]);
 #pragma unroll
-        for (int i = 0; i < MF; ++i) {
-          if (i < nfr) acc[i][f] = M::mma(af[i], bf, acc[i][f]);
-        }
+        for (int i = 0; i < NFR; ++i) acc[i][f] = M::mma(af[s & 1][i], bf, acc[i][f]);
       }
     }
+  };
+
+  issue(0);
+  for (int it = 0; it < n_kb; ++it) {
+    wait_dma();
+    __syncthreads();
+    if (it + 1 < n_kb) issue(it + 1);
+    compute(it);
   }
 
-  // ---- epilogue
+  // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
+  // column col0 + f.
   float flex = 1.0f;
   if (a.x_scale) flex *= *a.x_scale;
   if (a.w_scale) flex *= *a.w_scale;
   float bias[NF];
 #pragma unroll
   for (int f = 0; f < NF; ++f)
-    bias[f] = (a.bias && col[f] < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col[f])
-                                     : 0.f;
+    bias[f] = (a.bias && col0 + f < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col0 + f)
+                                       : 0.f;
   constexpr int NO = ACT == TAMD_ACT_SWIGLU ? NF / 2 : NF;  // outputs per lane per row
   const int n_out = ACT == TAMD_ACT_SWIGLU ? N / 2 : N;
-  const int out_col0 = ACT == TAMD_ACT_SWIGLU ? (t.n0 + wave * (16 * NF) + cidx * NF) / 2
-                                              : (t.n0 + wave * (16 * NF) + cidx * NF);
+  const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
   const bool has_limit = a.act_has_limit != 0;
 #pragma unroll
-  for (int i = 0; i < MF; ++i) {
-    if (i >= nfr) continue;
+  for (int i = 0; i < NFR; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int r = i * 16 + g * 4 + j;
+    for (int j = 0; j < 16; ++j) {
+      const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
       if (r >= t.rows) continue;
       const int erow = t.start_m + t.off_m + r;  // expert-sorted row
       int64_t dst = erow;
@@ -267,62 +324,81 @@ __global__ __launch_bounds__(256) void mm_x16_mxfp4_kernel(tamd_matmul_args a, i
       for (int f = 0; f < NF; ++f) v[f] = (acc[i][f][j] * flex + bias[f] * beta) * a.out_alpha;
       float o[NO];
       if constexpr (ACT == TAMD_ACT_SWIGLU) {
-#pragma unroll
-        for (int p = 0; p < NO; ++p) o[p] = swiglu_epi(v[2 * p], v[2 * p + 1], a.act_alpha, a.act_limit, has_limit);
+        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit) * gamma;
       } else {
 #pragma unroll
-        for (int p = 0; p < NO; ++p) o[p] = v[p];
+        for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
       }
       const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
       uint16_t *y16 = (uint16_t *)a.y + base + out_col0;
-      if (NO == 4 && a.y_dtype != TAMD_F32 && out_col0 + NO <= n_out && ((uintptr_t)y16 & 7) == 0) {
-        uint32_t lo, hi;
-        if (a.y_dtype == TAMD_BF16) {
-          lo = f32_to_bf16_bits(o[0] * gamma) | (f32_to_bf16_bits(o[1 % NO] * gamma) << 16);
-          hi = f32_to_bf16_bits(o[2 % NO] * gamma) | (f32_to_bf16_bits(o[3 % NO] * gamma) << 16);
-        } else {
-          lo = f32_to_f16_bits(o[0] * gamma) | (f32_to_f16_bits(o[1 % NO] * gamma) << 16);
-          hi = f32_to_f16_bits(o[2 % NO] * gamma) | (f32_to_f16_bits(o[3 % NO] * gamma) << 16);
-        }
-        *(uint2 *)y16 = make_uint2(lo, hi);
-      } else if (NO == 2 && a.y_dtype != TAMD_F32 && out_col0 + NO <= n_out && ((uintptr_t)y16 & 3) == 0) {
+      if (NO == 2 && a.y_dtype != TAMD_F32 && out_col0 + NO <= n_out && ((uintptr_t)y16 & 3) == 0) {
         uint32_t lo;
-        if (a.y_dtype == TAMD_BF16)
-          lo = f32_to_bf16_bits(o[0] * gamma) | (f32_to_bf16_bits(o[1 % NO] * gamma) << 16);
-        else
-          lo = f32_to_f16_bits(o[0] * gamma) | (f32_to_f16_bits(o[1 % NO] * gamma) << 16);
+        if (a.y_dtype == TAMD_BF16) lo = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[NO - 1]) << 16);
+        else lo = f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[NO - 1]) << 16);
         *(uint32_t *)y16 = lo;
       } else {
 #pragma unroll
         for (int p = 0; p < NO; ++p)
-          if (out_col0 + p < n_out) store_any(a.y, a.y_dtype, base + out_col0 + p, o[p] * gamma);
+          if (out_col0 + p < n_out) store_any(a.y, a.y_dtype, base + out_col0 + p, o[p]);
       }
     }
   }
 }
 
-template <int XDT, int MF, int NF>
-int launch_x16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int BLOCK_N = 64 * NF;
+// BM: block size of the ragged schedule the kernel consumes (16..128).
+template <int XDT, int BM, int ACT, bool SC_LDS>
+__global__ __launch_bounds__(256, 1) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+  constexpr int MF = BM <= 32 ? 1 : BM / 32;  // 32-row fragments
+  constexpr int LDS_ROWS = 32 * MF;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  Tile t;
+  if (!locate_tile<BM>(a, grid_n, grid_total, t)) return;
+  const int nfr = (t.rows + 31) / 32;  // active row fragments (workgroup uniform)
+#define TAMD_CASE(n)                                                           \
+  case n:                                                                      \
+    if constexpr (n <= MF) run_tile<XDT, n, LDS_ROWS, ACT, SC_LDS>(a, t, lds); \
+    break;
+  switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) }
+#undef TAMD_CASE
+}
+
+template <int XDT, int BM, int ACT>
+int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  constexpr int MF = BM <= 32 ? 1 : BM / 32;
+  constexpr int STAGE_BYTES = 32 * MF * ROW_BYTES + B_STAGE_BYTES;
   int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
   int64_t total = (int64_t)grid_m * grid_n;
   if (total <= 0) return 0;
   int64_t launch = ((total + 7) / 8) * 8;
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-  if (a.activation == TAMD_ACT_SWIGLU)
-    mm_x16_mxfp4_kernel<XDT, MF, NF, TAMD_ACT_SWIGLU><<<dim3((unsigned)launch), 256, 0, st>>>(a, grid_n, total);
-  else
-    mm_x16_mxfp4_kernel<XDT, MF, NF, TAMD_ACT_NONE><<<dim3((unsigned)launch), 256, 0, st>>>(a, grid_n, total);
+  // scales of a tile are staged in LDS when they are dense ([N][K/32]) and fit beside the stages
+  const int64_t G = a.K / 32;
+  const int64_t sc_bytes = (BLOCK_N * G + 15) / 16 * 16;
+  const bool dense_sc = a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
+                        aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0;
+  const int sc_in_lds = dense_sc && 2 * STAGE_BYTES + sc_bytes <= 160 * 1024;
+  const size_t lds_bytes = 2 * STAGE_BYTES + (sc_in_lds ? sc_bytes : 0);
+  auto kern = sc_in_lds ? mm_x16_mxfp4_kernel<XDT, BM, ACT, true> : mm_x16_mxfp4_kernel<XDT, BM, ACT, false>;
+  // raising the dynamic LDS limit is idempotent, so doing it on every launch keeps the entry point stateless
+  hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  kern<<<dim3((unsigned)launch), 256, lds_bytes, st>>>(a, grid_n, total);
   return launch_status();
+}
+
+template <int XDT, int BM>
+int launch_x16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  if (a.activation == TAMD_ACT_SWIGLU) return launch_x16_act<XDT, BM, TAMD_ACT_SWIGLU>(a, grid_m, st);
+  return launch_x16_act<XDT, BM, TAMD_ACT_NONE>(a, grid_m, st);
 }
 
 template <int XDT>
 int dispatch_x16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
   switch (block_m) {
-    case 16: return launch_x16<XDT, 1, 4>(a, grid_m, st);
-    case 32: return launch_x16<XDT, 2, 4>(a, grid_m, st);
-    case 64: return launch_x16<XDT, 4, 4>(a, grid_m, st);
-    case 128: return launch_x16<XDT, 8, 4>(a, grid_m, st);
+    case 16: return launch_x16<XDT, 16>(a, grid_m, st);
+    case 32: return launch_x16<XDT, 32>(a, grid_m, st);
+    case 64: return launch_x16<XDT, 64>(a, grid_m, st);
+    case 128: return launch_x16<XDT, 128>(a, grid_m, st);
     default: return TAMD_E_UNSUPPORTED;
   }
 }
@@ -353,6 +429,11 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     if (a.w_stride_k != 1 || a.w_mx_stride_k != 1) return TAMD_E_UNSUPPORTED;
     if (!aligned(a.w, 16) || a.w_stride_n % 16 != 0 || a.w_stride_e % 16 != 0) return TAMD_E_ALIGNMENT;
     if (!aligned(a.x, 16) || (a.x_stride_m * 2) % 16 != 0 || (a.x_stride_z * 2) % 16 != 0) return TAMD_E_ALIGNMENT;
+    // 32-bit buffer offsets: one batch of activations and one expert's weights must each span < 2 GiB
+    const int64_t x_rows = a.x_rows > 0 ? a.x_rows : a.M;
+    if (x_rows * a.x_stride_m * 2 >= (int64_t)0x7FFFFF00 || (int64_t)a.N * a.w_stride_n >= (int64_t)0x7FFFFF00 ||
+        (int64_t)a.N * a.w_mx_stride_n >= (int64_t)0x7FFFFF00)
+      return TAMD_E_UNSUPPORTED;
     int block_m, grid_m;
     if (ragged) {
       block_m = a.block_m;

@@ -223,6 +223,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     args.y, args.y_dtype = out.data_ptr(), _lib.dtype_code(out.dtype)
     args.y_stride_m, args.y_stride_z = out.stride(1), out.stride(0)
     args.M, args.N, args.K, args.n_experts = M, N, K, n_slices
+    args.x_rows = a.shape[-2]
     args.gather_indx, args.scatter_indx = i32(gather_indx), i32(scatter_indx)
     if ragged:
         md = a_ragged_metadata
