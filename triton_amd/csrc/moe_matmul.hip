@@ -33,8 +33,7 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-constexpr int KB = 128;            // K per pipeline stage
-constexpr int ROW_BYTES = KB * 2;  // LDS bytes per activation row per stage
+constexpr int KB = 128;  // K per weight (super-)stage
 constexpr int NF = 2;              // 32-column fragments per wave
 constexpr int BLOCK_N = 4 * 32 * NF;
 
@@ -157,23 +156,26 @@ TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
                __builtin_amdgcn_readfirstlane((int)((uint32_t)(p >> 32) & 0xFFFFu)), (int)num_records, 0x00020000};
 }
 
-constexpr int B_STAGE_BYTES = 4 * 64 * 64;  // 256 columns x 64 bytes (128 K of fp4) per stage
+constexpr int KA = 64;                 // K per activation stage
+constexpr int A_ROW_BYTES = KA * 2;    // LDS bytes per activation row per stage
+constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K of fp4)
 
-// One output tile with NFR (compile time) active 32-row fragments.  LDS: NSTAGE stages of
-// [A: LDS_ROWS x 256 B | B: 4 waves x 64 columns x 64 B], then the tile's e8m0 scales.
+// One output tile with NFR (compile time) active 32-row fragments.
+// LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | e8m0 scales of the tile].
 //
-// Both operands reach LDS by DMA, one stage ahead of the multiply.  Activations: thread (row
-// tid/16, slot tid%16) of every 16-row group fetches the 16-byte chunk slot^(row%16), so chunk c of
-// row r sits at slot c^(r%16) and the 32-row MFMA operand reads are bank-conflict free.  Weights:
-// each wave copies its own 64 columns, 64 contiguous bytes per column per stage (4 lanes x 16 B),
-// into position p' = f*32 + c (global column 2c + f of the wave's strip, so that a lane ends up
-// with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3 against conflicts.
+// Both operands reach LDS by DMA.  Activations: 64 K per stage, double buffered; wave w copies rows
+// 8w..8w+7 of every 32-row fragment (8 lanes x 16 B per row); chunk c of row r sits at slot
+// c ^ ((r>>1)&7), which makes the 32-row MFMA operand reads bank-conflict free.  Weights: every
+// second stage each wave copies 64 contiguous bytes (128 K) of each of its own 64 columns into
+// its private region, position p' = f*32 + c holding global column 2c + f of the wave's strip (so
+// a lane ends up with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3.
+// The wave reads them into registers at the start of the even stage and immediately requests the
+// next 128 K into the same region, so weights need no second buffer and no barrier.
 template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS>
 TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
-  constexpr int NG = 2 * NFR;  // 16-row groups staged per K stage
-  constexpr int STAGE_BYTES = LDS_ROWS * ROW_BYTES + B_STAGE_BYTES;
+  constexpr int A_STAGE = LDS_ROWS * A_ROW_BYTES;
   constexpr uint32_t kOob = 0x7FFFFFFFu;
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -184,7 +186,9 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
   const uint8_t *s_base = a.w_mx_scale + (int64_t)t.expert * a.w_mx_stride_e;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-  uint8_t *lds_sc = lds + 2 * STAGE_BYTES;
+  const uint32_t lds_b = lds_base + 2 * A_STAGE + wave * 4096;
+  const uint8_t *bbuf = lds + 2 * A_STAGE + wave * 4096;
+  uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES;
 
   // ---- scales of the whole tile, once: 256 columns x G bytes, contiguous in memory
   const int tile_cols = N - t.n0 < BLOCK_N ? N - t.n0 : BLOCK_N;
@@ -196,13 +200,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
   }
 
-  // ---- activation DMA: wave w copies rows 4w..4w+3 of every 16-row group
-  const int a_slot = lane % 16, a_row = wave * 4 + lane / 16;  // row inside a 16-row group
-  const int a_chunk = a_slot ^ a_row;
-  uint32_t a_off[NG];
+  // ---- activation DMA: one instruction per 32-row fragment, lane -> (row 8w + lane/8, slot lane%8)
+  const int a_rin = wave * 8 + lane / 8;
+  const int a_chunk = (lane % 8) ^ ((a_rin >> 1) & 7);
+  uint32_t a_off[NFR];
 #pragma unroll
-  for (int i = 0; i < NG; ++i) {
-    int r = i * 16 + a_row;
+  for (int i = 0; i < NFR; ++i) {
+    int r = i * 32 + a_rin;
     int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
     uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
     a_off[i] = src * (uint32_t)(a.x_stride_m * 2) + a_chunk * 16;
@@ -228,54 +232,61 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
       for (int j = 0; j < 16; ++j) acc[i][f][j] = 0.f;
 
-  const int n_kb = (K + KB - 1) / KB;
-  auto issue = [&](int it) {
-    const int kb = it * KB;
-    const uint32_t sb = lds_base + (it & 1) * STAGE_BYTES;
+  const int n_ka = (K + KA - 1) / KA;      // activation stages
+  const int n_kb = (K + KB - 1) / KB;      // weight super-stages (two activation stages each)
+  auto issue_a = [&](int it) {             // clamped: past the end the last stage is copied again
+    it = it < n_ka ? it : n_ka - 1;
+    const int kb = it * KA;
     const uint32_t akill = kb + a_chunk * 8 < K ? 0u : kOob;
+    const uint32_t sb = lds_base + (it & 1) * A_STAGE + wave * 8 * A_ROW_BYTES;
 #pragma unroll
-    for (int i = 0; i < NG; ++i) dma16(rx, sb + (i * 16 + wave * 4) * ROW_BYTES, a_off[i] | akill, kb * 2);
-    const uint32_t bb = sb + LDS_ROWS * ROW_BYTES + wave * 4096;
+    for (int i = 0; i < NFR; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * 2);
+  };
+  auto issue_b = [&](int sup) {
+    sup = sup < n_kb ? sup : n_kb - 1;
+    const int kb = sup * KB;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t bkill = kb + w_part[j] * 32 < K ? 0u : kOob;
-      dma16(rw, bb + j * 1024, w_off[j] | bkill, kb >> 1);
+      dma16(rw, lds_b + j * 1024, w_off[j] | bkill, kb >> 1);
     }
   };
 
-  auto compute = [&](int it) {
-    const uint8_t *buf = lds + (it & 1) * STAGE_BYTES;
-    const uint8_t *bbuf = buf + LDS_ROWS * ROW_BYTES + wave * 4096;
-    uint4 raw[NF][2];
-    float scf[NF][2];
+  uint4 raw[NF][2];
+  float scf[NF][2];
+  // registers <- this wave's weights and scales of super-stage `sup`
+  auto load_b = [&](int sup) {
 #pragma unroll
     for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int pos = f * 32 + c32;
-        raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * h + q) ^ ((pos >> 2) & 3)) * 16));
-        const int kg = it * 4 + 2 * h + q;
+        raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
+        const int kg = sup * 4 + 2 * q + h;
         uint32_t sbyte;
         if constexpr (SC_LDS) sbyte = lds_sc[(wave * 64 + c32 * NF + f) * G + (kg < G ? kg : G - 1)];
         else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + (kg < G ? kg : G - 1)];
         scf[f][q] = bits_to_f32(sbyte << 23);
       }
+  };
+
+  auto compute = [&](int it, auto qc) {
+    constexpr int q = decltype(qc)::value;
+    const uint8_t *buf = lds + (it & 1) * A_STAGE;
     auto read_frags = [&](int s, frag_t *af) {
-      const int chunk = h * 8 + (s >> 2) * 4 + (s & 3);
+      const int slot = (h * 4 + s) ^ ((c32 >> 1) & 7);
 #pragma unroll
-      for (int i = 0; i < NFR; ++i)
-        af[i] = *(const frag_t *)(buf + (i * 32 + c32) * ROW_BYTES + ((chunk ^ (c32 & 15)) * 16));
+      for (int i = 0; i < NFR; ++i) af[i] = *(const frag_t *)(buf + (i * 32 + c32) * A_ROW_BYTES + slot * 16);
     };
     frag_t af[2][NFR];
     read_frags(0, af[0]);
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      if (s < 7) read_frags(s + 1, af[(s + 1) & 1]);
-      const int q = s >> 2, u = s & 3;
+    for (int s = 0; s < 4; ++s) {
+      if (s < 3) read_frags(s + 1, af[(s + 1) & 1]);
 #pragma unroll
       for (int f = 0; f < NF; ++f) {
         const uint4 r = raw[f][q];
-        const uint32_t codes = u == 0 ? r.x : (u == 1 ? r.y : (u == 2 ? r.z : r.w));
+        const uint32_t codes = s == 0 ? r.x : (s == 1 ? r.y : (s == 2 ? r.z : r.w));
         const frag_t bf = M::expand(codes, scf[f][q]);
 #pragma unroll
         for (int i = 0; i < NFR; ++i) acc[i][f] = M::mma(af[s & 1][i], bf, acc[i][f]);
@@ -283,16 +294,28 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
   };
 
-  issue(0);
-  for (int it = 0; it < n_kb; ++it) {
+  issue_a(0);
+  issue_b(0);
+  for (int it = 0; it < n_ka; it += 2) {
     wait_dma();
     __syncthreads();
-    if (it + 1 < n_kb) issue(it + 1);
-    compute(it);
+    load_b(it >> 1);
+    issue_a(it + 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
+    issue_b((it >> 1) + 1);
+    compute(it, std::integral_constant<int, 0>{});
+    if (it + 1 < n_ka) {
+      wait_dma();
+      __syncthreads();
+      issue_a(it + 2);
+      compute(it + 1, std::integral_constant<int, 1>{});
+    }
   }
+  wait_dma();
 
   // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
-  // column col0 + f.
+  // column col0 + f.  16-bit outputs are staged through LDS (the K stages are dead by now) so
+  // that the global stores are 16 bytes per lane and whole rows of the tile are contiguous.
   float flex = 1.0f;
   if (a.x_scale) flex *= *a.x_scale;
   if (a.w_scale) flex *= *a.w_scale;
@@ -302,21 +325,20 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     bias[f] = (a.bias && col0 + f < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col0 + f)
                                        : 0.f;
   constexpr int NO = ACT == TAMD_ACT_SWIGLU ? NF / 2 : NF;  // outputs per lane per row
+  constexpr int OUT_COLS = 128 * NO;                        // output columns of the tile
   const int n_out = ACT == TAMD_ACT_SWIGLU ? N / 2 : N;
   const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
+  const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
   const bool has_limit = a.act_has_limit != 0;
+  const bool staged = a.y_dtype != TAMD_F32;
+  uint16_t *ob = (uint16_t *)lds;  // [rows][OUT_COLS]
+  __syncthreads();
 #pragma unroll
   for (int i = 0; i < NFR; ++i) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
-      if (r >= t.rows) continue;
-      const int erow = t.start_m + t.off_m + r;  // expert-sorted row
-      int64_t dst = erow;
-      if (a.scatter_indx) {
-        dst = a.scatter_indx[erow];
-        if (dst < 0) continue;
-      }
+      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
       const float beta = a.betas ? a.betas[erow] : 1.0f;
       const float gamma = a.gammas ? a.gammas[erow] : 1.0f;
       float v[NF];
@@ -329,17 +351,44 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
         for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
       }
-      const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
-      uint16_t *y16 = (uint16_t *)a.y + base + out_col0;
-      if (NO == 2 && a.y_dtype != TAMD_F32 && out_col0 + NO <= n_out && ((uintptr_t)y16 & 3) == 0) {
-        uint32_t lo;
-        if (a.y_dtype == TAMD_BF16) lo = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[NO - 1]) << 16);
-        else lo = f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[NO - 1]) << 16);
-        *(uint32_t *)y16 = lo;
-      } else {
+      if (staged) {
+        uint16_t *dstl = ob + r * OUT_COLS + wave * 32 * NO + c32 * NO;
+        if constexpr (NO == 2) {
+          uint32_t w2 = a.y_dtype == TAMD_BF16 ? (f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[NO - 1]) << 16))
+                                               : (f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[NO - 1]) << 16));
+          *(uint32_t *)dstl = w2;
+        } else {
+          *dstl = (uint16_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(o[0]) : f32_to_f16_bits(o[0]));
+        }
+      } else if (r < t.rows) {
+        int64_t dst = t.start_m + t.off_m + r;
+        if (a.scatter_indx) dst = a.scatter_indx[dst];
+        if (dst >= 0) {
+          const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
 #pragma unroll
-        for (int p = 0; p < NO; ++p)
-          if (out_col0 + p < n_out) store_any(a.y, a.y_dtype, base + out_col0 + p, o[p]);
+          for (int p = 0; p < NO; ++p)
+            if (out_col0 + p < n_out) ((float *)a.y)[base + out_col0 + p] = o[p];
+        }
+      }
+    }
+  }
+  if (staged) {
+    __syncthreads();
+    constexpr int CPR = OUT_COLS / 8;  // 16-byte chunks per tile row
+    const int n_chunks = t.rows * CPR;
+    for (int id = tid; id < n_chunks; id += 256) {
+      const int r = id / CPR, c = (id - r * CPR) * 8;
+      int64_t dst = t.start_m + t.off_m + r;
+      if (a.scatter_indx) dst = a.scatter_indx[dst];
+      if (dst < 0) continue;
+      const int gcol = tile_out0 + c;
+      if (gcol >= n_out) continue;
+      uint16_t *yp = (uint16_t *)a.y + (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol;
+      const uint16_t *sp = ob + r * OUT_COLS + c;
+      if (gcol + 8 <= n_out && ((uintptr_t)yp & 15) == 0) {
+        *(uint4 *)yp = *(const uint4 *)sp;
+      } else {
+        for (int e = 0; e < 8 && gcol + e < n_out; ++e) yp[e] = sp[e];
       }
     }
   }
@@ -347,7 +396,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 
 // BM: block size of the ragged schedule the kernel consumes (16..128).
 template <int XDT, int BM, int ACT, bool SC_LDS>
-__global__ __launch_bounds__(256, 1) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+__global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
   constexpr int MF = BM <= 32 ? 1 : BM / 32;  // 32-row fragments
   constexpr int LDS_ROWS = 32 * MF;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -365,19 +414,22 @@ __global__ __launch_bounds__(256, 1) void mm_x16_mxfp4_kernel(tamd_matmul_args a
 template <int XDT, int BM, int ACT>
 int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int MF = BM <= 32 ? 1 : BM / 32;
-  constexpr int STAGE_BYTES = 32 * MF * ROW_BYTES + B_STAGE_BYTES;
+  constexpr int LDS_ROWS = 32 * MF;
+  constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES;
+  constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
   int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
   int64_t total = (int64_t)grid_m * grid_n;
   if (total <= 0) return 0;
   int64_t launch = ((total + 7) / 8) * 8;
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-  // scales of a tile are staged in LDS when they are dense ([N][K/32]) and fit beside the stages
+  // scales of a tile are staged in LDS when they are dense ([N][K/32]) and two workgroups still fit a CU
   const int64_t G = a.K / 32;
   const int64_t sc_bytes = (BLOCK_N * G + 15) / 16 * 16;
   const bool dense_sc = a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
                         aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0;
-  const int sc_in_lds = dense_sc && 2 * STAGE_BYTES + sc_bytes <= 160 * 1024;
-  const size_t lds_bytes = 2 * STAGE_BYTES + (sc_in_lds ? sc_bytes : 0);
+  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;
+  size_t lds_bytes = PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
+  if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;
   auto kern = sc_in_lds ? mm_x16_mxfp4_kernel<XDT, BM, ACT, true> : mm_x16_mxfp4_kernel<XDT, BM, ACT, false>;
   // raising the dynamic LDS limit is idempotent, so doing it on every launch keeps the entry point stateless
   hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
