@@ -131,8 +131,13 @@ TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid
     t.start_m = 0;
     t.off_m = (pid_m - z * bm) * BLOCK_M;
   }
-  t.rows = slice_rows - t.off_m;
-  if (t.rows > BLOCK_M) t.rows = BLOCK_M;
+  // A 128-row block also takes a remainder of up to 32 rows that follows it (one more 32-row
+  // fragment), and that remainder's own block does nothing: with about 128 rows per expert this
+  // avoids a second, nearly empty pass over the expert's weights.
+  constexpr int EXTRA = BLOCK_M == 128 ? 32 : 0;
+  const int left = slice_rows - t.off_m;
+  if (EXTRA > 0 && t.off_m > 0 && left <= EXTRA) return false;
+  t.rows = left > BLOCK_M + EXTRA ? BLOCK_M : left;
   return t.rows > 0;
 }
 
@@ -397,7 +402,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 // BM: block size of the ragged schedule the kernel consumes (16..128).
 template <int XDT, int BM, int ACT, bool SC_LDS>
 __global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
-  constexpr int MF = BM <= 32 ? 1 : BM / 32;  // 32-row fragments
+  constexpr int MF = BM <= 32 ? 1 : (BM == 128 ? 5 : BM / 32);  // 32-row fragments (128 + 32 absorbed)
   constexpr int LDS_ROWS = 32 * MF;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   Tile t;
@@ -407,13 +412,13 @@ __global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a
   case n:                                                                      \
     if constexpr (n <= MF) run_tile<XDT, n, LDS_ROWS, ACT, SC_LDS>(a, t, lds); \
     break;
-  switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) }
+  switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) TAMD_CASE(5) }
 #undef TAMD_CASE
 }
 
 template <int XDT, int BM, int ACT>
 int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int MF = BM <= 32 ? 1 : BM / 32;
+  constexpr int MF = BM <= 32 ? 1 : (BM == 128 ? 5 : BM / 32);
   constexpr int LDS_ROWS = 32 * MF;
   constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES;
   constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
