@@ -1,0 +1,157 @@
+"""Pins oracle/matmul_ref.py (grouped matmul, SwiGLU, combine) with checks that a dropped term, a transposed
+operand or a wrong index would fail: float64 evaluation with python-level indexing on tiny shapes, one-hot
+activations that must reproduce dequantised weight rows bit for bit, zero weights that leave bias*beta*gamma,
+and limits of the activation."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import matmul_ref as MR
+from oracle import mxfp_ref as MX
+
+
+def _mx_weights(E, K, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(E, K, N, generator=g) * 0.5
+    q, s = MX.downcast_to_mxfp_ref(w, torch.uint8, axis=1)
+    return q, s, MX.upcast_from_mxfp_ref(q, s, torch.float32, axis=1)
+
+
+def test_dequantised_weights_are_exact_in_bf16():
+    # apply_precision dequantises to bf16 (matmul.py:772-778 of the reference); e2m1 * 2**e needs 2 mantissa bits
+    q, s, w32 = _mx_weights(2, 64, 8, 0)
+    w16 = MX.upcast_from_mxfp_ref(q, s, torch.bfloat16, axis=1)
+    assert torch.equal(w16.float(), w32)
+
+
+def test_ragged_gather_scatter_against_float64_loops():
+    torch.manual_seed(0)
+    E, K, N, T, k = 3, 64, 6, 5, 2
+    q, s, w = _mx_weights(E, K, N, 1)
+    x = torch.randn(T, K).bfloat16()
+    bias = torch.randn(E, N)
+    sizes = torch.tensor([4, 0, 6], dtype=torch.int32)
+    gather = torch.tensor([0, 1, 2, 4, 0, 1, 2, 3, 3, 4], dtype=torch.int32)
+    scatter = torch.tensor([3, 7, 1, 9, 0, 2, 4, 5, 6, 8], dtype=torch.int32)
+    betas = torch.rand(10)
+    gammas = torch.rand(10)
+    y = MR.matmul_ref(x, q, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=s,
+                      betas=betas, gammas=gammas)
+    assert y.dtype == torch.bfloat16 and y.shape == (10, N)
+    expert_of_row = [0] * 4 + [2] * 6
+    for r in range(10):
+        e = expert_of_row[r]
+        for n in range(N):
+            acc = 0.0
+            for kk in range(K):
+                acc += float(x[gather[r], kk]) * float(w[e, kk, n])
+            want = (acc + float(bias[e, n]) * float(betas[r])) * float(gammas[r])
+            got = float(y[scatter[r], n])
+            assert abs(got - want) <= 2**-8 * abs(want) + 1e-6, (r, n, got, want)
+
+
+def test_one_hot_rows_reproduce_weight_rows():
+    E, K, N = 2, 96, 10
+    q, s, w = _mx_weights(E, K, N, 2)
+    x = torch.zeros(6, K, dtype=torch.bfloat16)
+    hot = [0, 33, 95, 1, 64, 31]
+    for r, kk in enumerate(hot):
+        x[r, kk] = 1.0
+    y = MR.matmul_ref(x, q, None, slice_sizes=torch.tensor([3, 3], dtype=torch.int32), b_mx_scale=s)
+    for r, kk in enumerate(hot):
+        assert torch.equal(y[r].float(), w[r // 3, kk])  # a transposed or mis-grouped weight fails here
+
+
+def test_zero_weights_leave_bias_beta_gamma():
+    E, K, N = 2, 32, 4
+    q = torch.zeros(E, K // 2, N, dtype=torch.uint8)
+    s = torch.full((E, 1, N), 127, dtype=torch.uint8)
+    x = torch.randn(5, K).bfloat16()
+    bias = torch.tensor([[1.0, 2.0, 3.0, 4.0], [-1.0, -2.0, -3.0, -4.0]])
+    betas = torch.tensor([1.0, 0.5, 2.0, 0.0, 1.0])
+    gammas = torch.tensor([1.0, 1.0, 0.5, 3.0, -1.0])
+    y = MR.matmul_ref(x, q, bias, slice_sizes=torch.tensor([2, 3], dtype=torch.int32), b_mx_scale=s, betas=betas,
+                      gammas=gammas)
+    e_of = [0, 0, 1, 1, 1]
+    want = torch.stack([bias[e_of[r]] * betas[r] * gammas[r] for r in range(5)])
+    assert torch.equal(y.float(), want.bfloat16().float())
+
+
+def test_scatter_minus_one_drops_rows_and_flex_scale():
+    torch.manual_seed(3)
+    K, N = 32, 4
+    w = torch.randn(1, K, N)
+    x8 = (torch.randn(4, K)).to(torch.float8_e4m3fn)
+    sc = torch.tensor([0.25])
+    y = MR.matmul_ref(x8, w, None, slice_sizes=torch.tensor([4], dtype=torch.int32),
+                      scatter_indx=torch.tensor([2, -1, 0, 1], dtype=torch.int32), a_flex_scale=sc)
+    assert y.dtype == torch.float32  # fp8 + flex scale computes and returns float32 (matmul.py:761-764, 889)
+    full = (x8.double() * 0.25) @ w[0].double()
+    torch.testing.assert_close(y[2].double(), full[0], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(y[0].double(), full[2], rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(y[1].double(), full[3], rtol=1e-5, atol=1e-6)
+    assert y[3].eq(0).all()
+
+
+def test_dense_and_batched_modes():
+    torch.manual_seed(4)
+    a = torch.randn(3, 7, 16)
+    b = torch.randn(3, 16, 5)
+    bias = torch.randn(3, 5)
+    y = MR.matmul_ref(a, b, bias)
+    want = torch.einsum("bmk,bkn->bmn", a.double(), b.double()) + bias[:, None, :].double()
+    torch.testing.assert_close(y.double(), want, rtol=1e-5, atol=1e-5)
+    y2 = MR.matmul_ref(a[0], b[0], bias[0])
+    torch.testing.assert_close(y2, y[0])
+
+
+def test_swiglu_formula_float64_and_limits():
+    torch.manual_seed(5)
+    a = torch.randn(9, 16) * 4
+    alpha, limit = 1.702, 7.0
+    out = MR.swiglu_ref(a, alpha, limit)
+    for r in range(9):
+        for j in range(8):
+            g = min(float(a[r, 2 * j]), limit)          # gate: even column, clamped from above only
+            l = max(-limit, min(float(a[r, 2 * j + 1]), limit))
+            want = g / (1.0 + math.exp(-alpha * g)) * (l + 1.0)
+            assert abs(float(out[r, j]) - want) <= 1e-5 * max(1.0, abs(want))
+    far = torch.tensor([[-1e4, 3.0, 50.0, 2.0, 50.0, -50.0]])
+    o = MR.swiglu_ref(far, alpha, limit)
+    assert o[0, 0].item() == 0.0 or abs(o[0, 0].item()) < 1e-30      # g -> -inf gives 0 (not clamped below)
+    assert abs(o[0, 1].item() - 7.0 * (2.0 + 1.0)) < 1e-3             # large g saturates at limit, sigmoid -> 1
+    assert abs(o[0, 2].item() - 7.0 * (-7.0 + 1.0)) < 1e-3            # linear clamps on both sides
+    nolim = MR.swiglu_ref(far, alpha, None)
+    assert abs(nolim[0, 1].item() - 50.0 * 3.0) < 1e-3
+
+
+def test_fused_swiglu_order():
+    # kernel order: activation on the float32 result, then gamma, then the cast
+    torch.manual_seed(6)
+    K, N = 32, 8
+    w = torch.randn(1, K, N)
+    x = torch.randn(3, K).bfloat16()
+    gam = torch.tensor([0.5, 2.0, -1.0])
+    y = MR.matmul_ref(x, w, None, slice_sizes=torch.tensor([3], dtype=torch.int32), gammas=gam,
+                      fused_swiglu=(1.702, 7.0))
+    z = x.float() @ w[0]
+    want = (MR.swiglu_ref(z, 1.702, 7.0) * gam[:, None]).bfloat16()
+    assert torch.equal(y, want) and y.shape == (3, N // 2)
+
+
+def test_reduce_direct_sum():
+    torch.manual_seed(7)
+    x = torch.randn(6, 4, 10).bfloat16()
+    mask = torch.rand(6, 4, 1) > 0.3
+    scale = torch.rand(6, 4, 1)
+    z = MR.reduce_ref(x, 1, mask=mask, scale=scale)
+    for t in range(6):
+        for n in range(10):
+            acc = np.float32(0)
+            for j in range(4):
+                if mask[t, j, 0]:
+                    acc = np.float32(acc + np.float32(float(x[t, j, n])) * np.float32(float(scale[t, j, 0])))
+            assert float(z[t, n]) == float(torch.tensor(float(acc)).bfloat16()), (t, n)
+    assert torch.equal(MR.reduce_ref(x, 1), x.float().sum(1).bfloat16())
