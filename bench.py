@@ -28,7 +28,37 @@ WORKLOADS = {
     "fc1_decode": dict(T=64, E=128, k=4, K=2880, N=5760, act=True),
     # same rows and FLOPs as fc1_prefill with few experts: weights (66 MB) stay cache resident
     "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
+    # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
+    # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
+    "hbm_copy": dict(bytes=1 << 30),
 }
+
+
+def hbm_copy(args):
+    """dst = src * 1 over `bytes` of float32: reads and writes that many bytes once each."""
+    n = WORKLOADS["hbm_copy"]["bytes"] // 4
+    src = torch.ones(n, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    for _ in range(args.warmup):
+        torch.mul(src, 1.0, out=dst)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        torch.mul(src, 1.0, out=dst)
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    gbs = 2 * n * 4 / (ms * 1e-3) / 1e9
+    print(json.dumps({"metric": "hbm_copy_gbs", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": f"hbm_copy: torch.mul(src, 1.0, out=dst), {n * 4} bytes read + written"},
+                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel_ms": round(ms, 4)},
+                      "cpu_baseline": None}))
 
 
 def make_weights(E, K, N, device, seed=0):
@@ -92,6 +122,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
         sys.exit(3)
+
+    if args.workload == "hbm_copy":
+        hbm_copy(args)
+        return
 
     from oracle import routing_ref as RR
     from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
