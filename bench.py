@@ -20,7 +20,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
+PEAK_FP8_TFLOPS = 5000.0
 PEAK_MXFP4_TFLOPS = 10100.0
+
+# HBM bytes per launch of the dominant kernel (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00 KiB from rocprofv3 --pmc,
+# factors from the hbm_copy workload).  Counters cannot be read from inside this process; re-measure after kernel changes.
+MEASURED_TRAFFIC = {"fc1_prefill": 1536778240, "fc1_decode": 1558978560}
 
 WORKLOADS = {
     # name: (T, E, k, K, N, swiglu)
@@ -28,6 +33,8 @@ WORKLOADS = {
     "fc1_decode": dict(T=64, E=128, k=4, K=2880, N=5760, act=True),
     # same rows and FLOPs as fc1_prefill with few experts: weights (66 MB) stay cache resident
     "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
+    # down projection + combine: fp8 (per-tensor scaled) expert-sorted rows x MXFP4 W2, gate weights, scatter, k-way sum
+    "fc2_combine": dict(T=16384, E=32, k=4, K=2880, N=2880, act=False, fc2=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
     # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
     "hbm_copy": dict(bytes=1 << 30),
@@ -88,22 +95,121 @@ def algorithmic_bytes(col_sum, T, k, K, N, act):
     return rows * K * 2 + rows * n_out * 2 + n_active * per_expert, n_active
 
 
-def cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, experts, K, N, act):
+def cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, experts, K, N, act, fc2=None):
     """Oracle (CPU restatement of the reference's torch path) timed on a bounded sample: the first
-    `experts` experts of the same workload, all host cores."""
+    `experts` experts of the same workload, all host cores.  For the down projection `fc2` holds
+    (x_scale, gammas) and the rows are already expert-sorted."""
     from oracle import matmul_ref as MR
     torch.set_num_threads(os.cpu_count())
     sizes = ref["col_sum"][:experts]
     n_rows = int(sizes.sum())
-    gather = ref["gather_indx"][:n_rows]
     v = vals[:experts].cpu()
     s = scales[:experts].cpu()
     t0 = time.perf_counter()
-    y = MR.matmul_ref(x_cpu, v, bias_cpu[:experts], slice_sizes=sizes, gather_indx=gather, b_mx_scale=s,
-                      fused_swiglu=(1.702, 7.0) if act else None)
+    if fc2 is None:
+        gather = ref["gather_indx"][:n_rows]
+        y = MR.matmul_ref(x_cpu, v, bias_cpu[:experts], slice_sizes=sizes, gather_indx=gather, b_mx_scale=s,
+                          fused_swiglu=(1.702, 7.0) if act else None)
+    else:
+        x_scale, gammas = fc2
+        y = MR.matmul_ref(x_cpu[:n_rows], v, bias_cpu[:experts], slice_sizes=sizes, b_mx_scale=s, a_flex_scale=x_scale,
+                          gammas=gammas[:n_rows]).to(torch.bfloat16)
     dt = time.perf_counter() - t0
     flops = 2.0 * n_rows * K * N
     return y, n_rows, flops / dt / 1e12, dt
+
+
+def run_fc2(args, cfg):
+    """BASELINE config 5: y = scatter((x8 . deq(W2[e]) * sx + bias[e]) * gate), z = sum over the k slots."""
+    from oracle import routing_ref as RR
+    from triton_amd.matmul import FlexCtx, InFlexData, PrecisionConfig, matmul
+    from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
+    from triton_amd.reduce import reduce
+    from triton_amd.routing import routing
+    T, E, k, K, N = cfg["T"], cfg["E"], cfg["k"], cfg["K"], cfg["N"]
+    rows = T * k
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    logits_cpu = torch.randn(T, E)
+    bias_cpu = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    x0 = torch.randn((rows, K), generator=g, device=dev, dtype=torch.float32)
+    x_scale = (x0.abs().max() / 448.0).reshape(1)
+    x8 = (x0 / x_scale).to(torch.float8_e4m3fn)
+    del x0
+    logits, bias = logits_cpu.to(dev), bias_cpu.to(dev)
+    vals, scales = make_weights(E, K, N, dev)
+    pc = PrecisionConfig(b_mx_scale=scales, b_microblock_size=32, out_dtype=torch.bfloat16,
+                         flex_ctx=FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale)))
+    y_buf = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
+    constraints = {"block_m": args.block_m} if args.block_m else {}
+
+    def step(ev=None):
+        r = routing(logits, k)
+        gam = r.expert_sorted_gate_weights
+        if ev is not None:
+            ev[0].record()
+        y = matmul(x8, vals, bias, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam, c=y_buf)
+        if ev is not None:
+            ev[1].record()
+        z, _ = reduce(y.view(T, k, N), dim=1)
+        return r, gam, y, z
+
+    with scoped_opt_flags_constraints(constraints):
+        for _ in range(args.warmup):
+            r, gam, y, z = step()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            r, gam, y, z = step(events[i])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    flops = 2.0 * rows * K * N
+    col_sum = r.col_sum.cpu()
+    n_active = int((col_sum > 0).sum())
+    mm_bytes = rows * K + n_active * (K // 2 * N + K // 32 * N + N * 2) + rows * 8 + rows * N * 2
+    tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
+    roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_FP8_TFLOPS, unit="TFLOP/s",
+                frac=round(tflops_kernel / PEAK_FP8_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
+                kernel="mm_x8_mxfp4_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
+                algorithmic_flops=flops, frac_of_mxfp4_peak=round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4),
+                hbm_gbs=round(mm_bytes / (kernel_ms * 1e-3) / 1e9, 1))
+    ref = RR.routing_ref(logits_cpu, k)
+    routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(col_sum, ref["col_sum"]))
+    gam_ref = ref["vals"].flatten()[ref["col_sorted_indx"].long()]
+    routing_ok = routing_ok and bool(torch.allclose(gam.cpu(), gam_ref, rtol=1e-5, atol=1e-7))  # softmax values
+    gam_ref = gam.cpu()
+    # the combine is a fixed-order fp32 sum: bit-exact given y
+    from oracle import matmul_ref as MR
+    n_chk = 2048
+    combine_ok = bool(torch.equal(z[:n_chk].cpu(), MR.reduce_ref(y.view(T, k, N)[:n_chk].cpu(), 1)))
+    cpu, gemm_ok = None, None
+    if args.cpu_experts > 0:
+        n_e = min(args.cpu_experts, E)
+        y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x8.cpu(), vals, scales, bias_cpu, ref, n_e, K, N, False,
+                                                        fc2=(x_scale.cpu(), gam_ref))
+        got = y.cpu()[ref["scatter_indx"][:n_rows].long()]
+        gemm_ok = bool(torch.allclose(got.float(), y_ref.float(), rtol=1e-2, atol=1e-2))
+        cpu = dict(value=round(cpu_tflops, 5), unit="TFLOP/s", cores=os.cpu_count(), kind="port",
+                   sample=f"oracle matmul_ref (dequantise + fp32 GEMM, gate weights) on the first {n_e} of {E} experts "
+                          f"({n_rows} of {rows} rows), {cpu_s:.1f} s")
+    print(json.dumps({
+        "metric": "moe_matmul_ogs_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8e4m3 x mxfp4 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: routing + matmul_ogs(fp8 rows, grouped GEMM, bias, gate weights, scatter) + "
+                               f"top-{k} combine, T={T}, hidden={K}, experts={E}, W2 mxfp4 [{E},{K},{N}]",
+                   "rows": rows, "active_experts": n_active},
+        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
+        "roofline": roof, "cpu_baseline": cpu,
+        "parity": {"routing_bit_exact": routing_ok, "combine_bit_exact": combine_ok, "gemm_sample_within_1e-2": gemm_ok},
+    }))
 
 
 def main():
@@ -125,6 +231,10 @@ def main():
 
     if args.workload == "hbm_copy":
         hbm_copy(args)
+        return
+
+    if WORKLOADS[args.workload].get("fc2"):
+        run_fc2(args, WORKLOADS[args.workload])
         return
 
     from oracle import routing_ref as RR
@@ -182,10 +292,10 @@ def main():
     hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (PEAK_BF16_TFLOPS * 1e12))
     if hbm_bound:
         roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=None)
+                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
     else:
         roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=round(tflops_kernel / PEAK_BF16_TFLOPS, 4), traffic=None)
+                    frac=round(tflops_kernel / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
     roof["kernel"] = "mm_x16_mxfp4_kernel"
     roof["kernel_ms"] = round(kernel_ms, 4)
     roof["algorithmic_bytes"] = abytes

@@ -7,7 +7,7 @@ import torch
 from oracle import matmul_ref as MR
 from oracle import routing_ref as RR
 from oracle.mxfp_ref import downcast_to_mxfp_ref
-from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul, matmul_ogs
+from triton_amd.matmul import FlexCtx, FnSpecs, FusedActivation, InFlexData, PrecisionConfig, matmul, matmul_ogs
 from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
 from triton_amd.numerics_details.mxfp import downcast_to_mxfp
 from triton_amd.routing import routing
@@ -153,3 +153,104 @@ def test_empty(device):
     out = matmul(torch.empty((0, 64), dtype=torch.bfloat16, device=device), w, None,
                  precision_config=PrecisionConfig(b_mx_scale=s, b_microblock_size=32))
     assert tuple(out.shape) == (0, 64)
+
+
+# ---------------------------------------------------------------------------- fp8 activations (scaled MFMA)
+
+
+def to_fp8(x0):
+    """Per-tensor flex quantisation as in BASELINE config 5: s = amax / 448, x = (x0 / s) -> e4m3."""
+    s = x0.abs().max() / 448.0
+    return (x0 / s).to(torch.float8_e4m3fn), s.reshape(1).float()
+
+
+def fp8_pc(s_w, x_scale, device, out_dtype):
+    flex = FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale.to(device)))
+    return PrecisionConfig(b_mx_scale=s_w, b_microblock_size=32, flex_ctx=flex, out_dtype=out_dtype)
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 2048, 512), (16, 64, 64), (33, 96, 200), (130, 192, 520), (1, 32, 16),
+                                   (128, 2880, 256)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_fp8_dense(M, K, N, out_dtype, device):
+    torch.manual_seed(0)
+    x8, xs = to_fp8(torch.randn(M, K))
+    w = torch.randn(K, N) * 0.02
+    bias = torch.randn(N) * 0.1
+    v, s, rv, rs = quantize_w(w, device)
+    out = matmul(x8.to(device), v, bias.to(device), precision_config=fp8_pc(s, xs, device, out_dtype))
+    ref = MR.matmul_ref(x8, rv, bias, b_mx_scale=rs, a_flex_scale=xs)
+    assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+    check(out, ref.to(out_dtype))
+
+
+def test_fp8_one_hot_rows_are_exact(device):
+    """x = one-hot rows (1.0 is exact in e4m3): the scaled MFMA must return the dequantised weight rows bit for
+    bit, which pins the K order of both operands and the scale-byte selection."""
+    torch.manual_seed(1)
+    K, N = 256, 256
+    w = torch.randn(K, N)
+    v, s, rv, rs = quantize_w(w, device)
+    x8 = torch.eye(K)[:160].to(torch.float8_e4m3fn)
+    one = torch.ones(1)
+    out = matmul(x8.to(device), v, None, precision_config=fp8_pc(s, one, device, torch.float32))
+    from oracle.mxfp_ref import upcast_from_mxfp_ref
+    deq = upcast_from_mxfp_ref(rv, rs, torch.float32, axis=0)
+    assert torch.equal(out.cpu(), deq[:160])
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128])
+@pytest.mark.parametrize("do_gather,do_scatter,do_gamma,act", [(False, False, False, False), (True, False, False, True),
+                                                                (False, True, True, False)])
+def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, device):
+    torch.manual_seed(0)
+    E, K, N, M = 9, 320, 392, 700
+    sizes = torch.tensor([0, 5, 130, 16, 1, 257, 64, 200, 27], dtype=torch.int32)
+    x8, xs = to_fp8(torch.randn(M, K))
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    gather = torch.randint(0, M, (M, ), dtype=torch.int32) if do_gather else None
+    scatter = torch.randperm(M, dtype=torch.int32) if do_scatter else None
+    if do_scatter:
+        scatter[::13] = -1
+    gammas = 2.0**torch.randint(-5, 0, (M, )).float() if do_gamma else None
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    dev = lambda t: None if t is None else t.to(device)
+    fa = swiglu_act(1.702, 7.0) if act else None
+    out_init = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=device)
+    with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+        out = matmul(dev(x8), v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter),
+                     precision_config=fp8_pc(s, xs, device, torch.bfloat16), gammas=dev(gammas), fused_activation=fa,
+                     c=out_init)
+    ref = MR.matmul_ref(x8, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs,
+                        a_flex_scale=xs, gammas=gammas, fused_swiglu=(1.702, 7.0) if act else None)
+    check(out, ref.to(torch.bfloat16))
+
+
+def test_moe_down_projection_and_combine_small(device):
+    """Config-5-shaped pipeline at reduced size: expert-sorted fp8 rows -> grouped GEMM * gate weights ->
+    scatter to (token, slot) order -> top-k combine."""
+    from triton_amd.reduce import reduce
+    torch.manual_seed(0)
+    T, E, k, H = 256, 8, 4, 2880
+    N = 384
+    logits = torch.randn(T, E)
+    r = routing(logits.to(device), k)
+    rr = RR.routing_ref(logits, k)
+    x8, xs = to_fp8(torch.randn(T * k, H))
+    w = torch.randn(E, H, N) * 0.02
+    bias = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
+    v, s, rv, rs = quantize_w(w, device)
+    gam = r.expert_sorted_gate_weights
+    gam_ref = rr["vals"].flatten()[rr["col_sorted_indx"].long()]
+    torch.testing.assert_close(gam.cpu(), gam_ref, rtol=1e-5, atol=1e-7)  # softmax values: exp is not bit-pinned
+    gam_ref = gam.cpu()
+    y = matmul(x8.to(device), v, bias.to(device), r.ragged_metadata, scatter_indx=r.scatter_indx,
+               precision_config=fp8_pc(s, xs, device, torch.bfloat16), gammas=gam)
+    y_ref = MR.matmul_ref(x8, rv, bias, slice_sizes=rr["col_sum"], scatter_indx=rr["scatter_indx"], b_mx_scale=rs,
+                          a_flex_scale=xs, gammas=gam_ref).to(torch.bfloat16)
+    check(y, y_ref)
+    z, _ = reduce(y.view(T, k, N), dim=1)
+    z_ref = MR.reduce_ref(y.cpu().view(T, k, N), 1)
+    assert torch.equal(z.cpu(), z_ref)  # fixed summation order: the combine is bit-exact given y

@@ -10,7 +10,8 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtriton_amd.so")
-SOURCES = ["api.cpp", "mxfp.hip", "routing.hip", "elementwise.hip", "moe_matmul.hip", "moe_matmul_fp8.hip"]
+SOURCES = ["api.cpp", "mxfp.hip", "routing.hip", "elementwise.hip", "moe_matmul.hip", "moe_matmul_bf16.hip", "moe_matmul_f16.hip",
+           "moe_matmul_fp8.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 math is switched off on purpose (device code only)
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
@@ -30,7 +31,8 @@ def build(force=True, verbose=False):
     os.makedirs(objdir, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in srcs]
-    deps = [os.path.join(CSRC, "common.h"), os.path.join(HERE, "..", "include", "triton_amd.h")]
+    deps = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "moe_matmul_impl.h"),
+            os.path.join(HERE, "..", "include", "triton_amd.h")]
     todo = []
     for s, o in zip(srcs, objs):
         newest = max(os.path.getmtime(p) for p in [os.path.join(CSRC, s), *deps])

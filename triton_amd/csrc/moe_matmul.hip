@@ -1,465 +1,12 @@
-// Grouped (ragged-M) / dense matmul for gfx950: 16-bit activations x MXFP4 weights.
-//
-//   y[dst(r), :] = act(((x[src(r), :] . deq(w[e])) * sx * sw + bias[e, :] * beta[r]) * alpha) * gamma[r]
-//
-// (matmul_details/_matmul.py:43-669 of the reference; epilogue order :540-559.)
-//
-// Work decomposition
-//   workgroup (4 waves) = one BLOCK_M x 256 output tile of one expert, taken from the ragged
-//     block schedule ((block << 16) | expert, -1 = padding);
-//   wave w owns the 64 columns [64w, 64w+64) of the tile and ALL its rows: the MXFP4 weights
-//     of those columns go HBM -> registers (one 128-bit load = 32 consecutive K of one column =
-//     one e8m0 group), are expanded to bf16/f16 in registers with v_cvt_scalef32_pk_*_fp4 and
-//     feed v_mfma_f32_32x32x16 as the B operand, so every weight byte is fetched and converted
-//     once per workgroup and never touches LDS;
-//   the activation rows (gathered) are staged through LDS, double buffered, 128 K per stage,
-//     16-byte chunks XOR-swizzled by row so that the MFMA A-operand reads hit distinct banks.
-//
-// The 32x32x16 MFMA is used because it sustains twice the rate of 16x16x32 on this part
-// (measured 2.45 vs 1.25 PFLOP/s for bf16).
-//
-// K order inside a 128-K stage: lane half h = lane/32 holds K [64q + 32h, 64q + 32h + 32) of its
-// column for q = 0, 1 (two 128-bit loads); MFMA step s = 4q + u consumes elements [8u, 8u+8) of
-// load q in both halves, for A and B alike.
-#include <type_traits>
-
+// C ABI entry point of the grouped / dense matmul: validation and dispatch.  The kernels live in
+// moe_matmul_impl.h and are instantiated once per activation type in moe_matmul_{bf16,f16,fp8}.hip
+// (separate translation units so that they compile in parallel).
 #include "common.h"
 
 namespace tamd {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
-
-constexpr int KB = 128;  // K per weight (super-)stage
-constexpr int NF = 2;              // 32-column fragments per wave
-constexpr int BLOCK_N = 4 * 32 * NF;
-
-template <int XDT>
-struct Mma;
-template <>
-struct Mma<TAMD_BF16> {
-  typedef bf16x8_t frag_t;
-  static TAMD_DEVICE frag_t expand(uint32_t codes, float scale) {
-    bf16x2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 0);
-    bf16x2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 1);
-    bf16x2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 2);
-    bf16x2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(codes, scale, 3);
-    return frag_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-  }
-  static TAMD_DEVICE f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mma<TAMD_F16> {
-  typedef f16x8_t frag_t;
-  static TAMD_DEVICE frag_t expand(uint32_t codes, float scale) {
-    f16x2_t p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, scale, 0);
-    f16x2_t p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, scale, 1);
-    f16x2_t p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, scale, 2);
-    f16x2_t p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, scale, 3);
-    return frag_t{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-  }
-  static TAMD_DEVICE f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-};
-
-TAMD_DEVICE float load_any_f32(const void *p, int dt, int64_t i) {
-  if (dt == TAMD_F32) return ((const float *)p)[i];
-  if (dt == TAMD_BF16) return bf16_bits_to_f32(((const uint16_t *)p)[i]);
-  return f16_bits_to_f32(((const uint16_t *)p)[i]);
-}
-
-TAMD_DEVICE void store_any(void *p, int dt, int64_t i, float v) {
-  if (dt == TAMD_F32) ((float *)p)[i] = v;
-  else if (dt == TAMD_BF16) ((uint16_t *)p)[i] = (uint16_t)f32_to_bf16_bits(v);
-  else ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v);
-}
-
-// Gate for the fused epilogue (swiglu_details/_swiglu.py:55-65): exp and reciprocal on the
-// hardware transcendental unit (relative error ~1e-6, far inside the 16-bit output rounding).
-TAMD_DEVICE float swiglu_fast(float g, float l, float alpha, float limit, bool has_limit) {
-  if (has_limit) {
-    g = __builtin_fminf(g, limit);
-    l = __builtin_fminf(__builtin_fmaxf(l, -limit), limit);
-  }
-  float e = __builtin_amdgcn_exp2f(-alpha * 1.4426950408889634f * g);
-  float s = g * __builtin_amdgcn_rcpf(1.0f + e);
-  return __builtin_fmaf(s, l, s);
-}
-
-// Tile coordinates of a workgroup.
-struct Tile {
-  int expert;   // weight slice
-  int z;        // batch index (dense batched) else 0
-  int start_m;  // first expert-sorted row of the slice
-  int off_m;    // first row of the tile inside the slice
-  int rows;     // valid rows in the tile (1..BLOCK_M)
-  int n0;       // first column of the tile
-};
-
-template <int BLOCK_M>
-TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid_total, Tile &t) {
-  // XCD-aware remap: hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
-  // contiguous range of tiles so neighbours (same expert, adjacent columns) share one L2.
-  const int64_t per_xcd = (grid_total + 7) / 8;
-  int64_t pid = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (pid >= grid_total) return false;
-  int pid_m = (int)(pid / grid_n);
-  int pid_n = (int)(pid - (int64_t)pid_m * grid_n);
-  t.n0 = pid_n * BLOCK_N;
-  t.z = 0;
-  int slice_rows;
-  if (a.block_schedule) {
-    int sched = a.block_schedule[pid_m];
-    if (sched == -1) return false;
-    t.expert = sched & 0xFFFF;
-    int blk = sched >> 16;
-    slice_rows = a.slice_sizes[t.expert];
-    t.start_m = a.slice_offs[t.expert];
-    t.off_m = blk * BLOCK_M;
-  } else {
-    int bm = (a.M + BLOCK_M - 1) / BLOCK_M;
-    int z = pid_m / bm;
-    t.expert = z;
-    t.z = z;
-    slice_rows = a.M;
-    t.start_m = 0;
-    t.off_m = (pid_m - z * bm) * BLOCK_M;
-  }
-  // A 128-row block also takes a remainder of up to 32 rows that follows it (one more 32-row
-  // fragment), and that remainder's own block does nothing: with about 128 rows per expert this
-  // avoids a second, nearly empty pass over the expert's weights.
-  constexpr int EXTRA = BLOCK_M == 128 ? 32 : 0;
-  const int left = slice_rows - t.off_m;
-  if (EXTRA > 0 && t.off_m > 0 && left <= EXTRA) return false;
-  t.rows = left > BLOCK_M + EXTRA ? BLOCK_M : left;
-  return t.rows > 0;
-}
-
-// 128-bit global -> LDS copy that bypasses registers (buffer_load ... lds).  The LDS destination of
-// lane L is lds_addr + 16*L; out-of-range offsets (>= num_records of the descriptor) deliver zeros.
-// Issued through inline asm so that the compiler does not serialise later LDS reads behind it; the
-// kernel waits for these copies itself (wait_dma) before the barrier that publishes a stage.
-typedef int v4i_t __attribute__((ext_vector_type(4)));
-TAMD_DEVICE void dma16(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :
-               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
-                 "s"(__builtin_amdgcn_readfirstlane(soff))
-               : "memory", "m0");
-}
-TAMD_DEVICE void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
-  uint64_t p = (uint64_t)base;
-  return v4i_t{__builtin_amdgcn_readfirstlane((int)(uint32_t)p),
-               __builtin_amdgcn_readfirstlane((int)((uint32_t)(p >> 32) & 0xFFFFu)), (int)num_records, 0x00020000};
-}
-
-constexpr int KA = 64;                 // K per activation stage
-constexpr int A_ROW_BYTES = KA * 2;    // LDS bytes per activation row per stage
-constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K of fp4)
-
-// One output tile with NFR (compile time) active 32-row fragments.
-// LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | e8m0 scales of the tile].
-//
-// Both operands reach LDS by DMA.  Activations: 64 K per stage, double buffered; wave w copies rows
-// 8w..8w+7 of every 32-row fragment (8 lanes x 16 B per row); chunk c of row r sits at slot
-// c ^ ((r>>1)&7), which makes the 32-row MFMA operand reads bank-conflict free.  Weights: every
-// second stage each wave copies 64 contiguous bytes (128 K) of each of its own 64 columns into
-// its private region, position p' = f*32 + c holding global column 2c + f of the wave's strip (so
-// a lane ends up with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3.
-// The wave reads them into registers at the start of the even stage and immediately requests the
-// next 128 K into the same region, so weights need no second buffer and no barrier.
-template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS>
-TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds) {
-  typedef Mma<XDT> M;
-  typedef typename M::frag_t frag_t;
-  constexpr int A_STAGE = LDS_ROWS * A_ROW_BYTES;
-  constexpr uint32_t kOob = 0x7FFFFFFFu;
-  const int tid = threadIdx.x;
-  const int wave = tid / kWave, lane = tid % kWave;
-  const int c32 = lane % 32, h = lane / 32;
-  const int K = a.K, N = a.N, G = K / 32;
-
-  const v4i_t rx = make_rsrc((const uint8_t *)a.x + (int64_t)t.z * a.x_stride_z * 2, kOob);
-  const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
-  const uint8_t *s_base = a.w_mx_scale + (int64_t)t.expert * a.w_mx_stride_e;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-  const uint32_t lds_b = lds_base + 2 * A_STAGE + wave * 4096;
-  const uint8_t *bbuf = lds + 2 * A_STAGE + wave * 4096;
-  uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES;
-
-  // ---- scales of the whole tile, once: 256 columns x G bytes, contiguous in memory
-  const int tile_cols = N - t.n0 < BLOCK_N ? N - t.n0 : BLOCK_N;
-  if constexpr (SC_LDS) {
-    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(s_base + (int64_t)t.n0 * G), 0, (uint32_t)(tile_cols * G), 0x00020000);
-    const int n_dw = (BLOCK_N * G + 3) / 4;
-    for (int i = tid; i < n_dw; i += 256)
-      ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
-  }
-
-  // ---- activation DMA: one instruction per 32-row fragment, lane -> (row 8w + lane/8, slot lane%8)
-  const int a_rin = wave * 8 + lane / 8;
-  const int a_chunk = (lane % 8) ^ ((a_rin >> 1) & 7);
-  uint32_t a_off[NFR];
-#pragma unroll
-  for (int i = 0; i < NFR; ++i) {
-    int r = i * 32 + a_rin;
-    int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
-    uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
-    a_off[i] = src * (uint32_t)(a.x_stride_m * 2) + a_chunk * 16;
-  }
-  // ---- weight DMA: instruction j copies LDS positions j*16 + lane/4, part slot lane%4
-  uint32_t w_off[4];
-  int w_part[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int pos = j * 16 + lane / 4;  // f*32 + c
-    const int col = t.n0 + wave * 64 + 2 * (pos % 32) + pos / 32;
-    w_part[j] = (lane % 4) ^ ((pos >> 2) & 3);
-    w_off[j] = (uint32_t)(col < N ? col : N - 1) * (uint32_t)a.w_stride_n + w_part[j] * 16;
-  }
-  // ---- this lane's MFMA columns
-  const int col0 = t.n0 + wave * 64 + c32 * NF;
-
-  f32x16_t acc[NFR][NF];
-#pragma unroll
-  for (int i = 0; i < NFR; ++i)
-#pragma unroll
-    for (int f = 0; f < NF; ++f)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) acc[i][f][j] = 0.f;
-
-  const int n_ka = (K + KA - 1) / KA;      // activation stages
-  const int n_kb = (K + KB - 1) / KB;      // weight super-stages (two activation stages each)
-  auto issue_a = [&](int it) {             // clamped: past the end the last stage is copied again
-    it = it < n_ka ? it : n_ka - 1;
-    const int kb = it * KA;
-    const uint32_t akill = kb + a_chunk * 8 < K ? 0u : kOob;
-    const uint32_t sb = lds_base + (it & 1) * A_STAGE + wave * 8 * A_ROW_BYTES;
-#pragma unroll
-    for (int i = 0; i < NFR; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * 2);
-  };
-  auto issue_b = [&](int sup) {
-    sup = sup < n_kb ? sup : n_kb - 1;
-    const int kb = sup * KB;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t bkill = kb + w_part[j] * 32 < K ? 0u : kOob;
-      dma16(rw, lds_b + j * 1024, w_off[j] | bkill, kb >> 1);
-    }
-  };
-
-  uint4 raw[NF][2];
-  float scf[NF][2];
-  // registers <- this wave's weights and scales of super-stage `sup`
-  auto load_b = [&](int sup) {
-#pragma unroll
-    for (int f = 0; f < NF; ++f)
-#pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const int pos = f * 32 + c32;
-        raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
-        const int kg = sup * 4 + 2 * q + h;
-        uint32_t sbyte;
-        if constexpr (SC_LDS) sbyte = lds_sc[(wave * 64 + c32 * NF + f) * G + (kg < G ? kg : G - 1)];
-        else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + (kg < G ? kg : G - 1)];
-        scf[f][q] = bits_to_f32(sbyte << 23);
-      }
-  };
-
-  auto compute = [&](int it, auto qc) {
-    constexpr int q = decltype(qc)::value;
-    const uint8_t *buf = lds + (it & 1) * A_STAGE;
-    auto read_frags = [&](int s, frag_t *af) {
-      const int slot = (h * 4 + s) ^ ((c32 >> 1) & 7);
-#pragma unroll
-      for (int i = 0; i < NFR; ++i) af[i] = *(const frag_t *)(buf + (i * 32 + c32) * A_ROW_BYTES + slot * 16);
-    };
-    frag_t af[2][NFR];
-    read_frags(0, af[0]);
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (s < 3) read_frags(s + 1, af[(s + 1) & 1]);
-#pragma unroll
-      for (int f = 0; f < NF; ++f) {
-        const uint4 r = raw[f][q];
-        const uint32_t codes = s == 0 ? r.x : (s == 1 ? r.y : (s == 2 ? r.z : r.w));
-        const frag_t bf = M::expand(codes, scf[f][q]);
-#pragma unroll
-        for (int i = 0; i < NFR; ++i) acc[i][f] = M::mma(af[s & 1][i], bf, acc[i][f]);
-      }
-    }
-  };
-
-  issue_a(0);
-  issue_b(0);
-  for (int it = 0; it < n_ka; it += 2) {
-    wait_dma();
-    __syncthreads();
-    load_b(it >> 1);
-    issue_a(it + 1);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
-    issue_b((it >> 1) + 1);
-    compute(it, std::integral_constant<int, 0>{});
-    if (it + 1 < n_ka) {
-      wait_dma();
-      __syncthreads();
-      issue_a(it + 2);
-      compute(it + 1, std::integral_constant<int, 1>{});
-    }
-  }
-  wait_dma();
-
-  // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
-  // column col0 + f.  16-bit outputs are staged through LDS (the K stages are dead by now) so
-  // that the global stores are 16 bytes per lane and whole rows of the tile are contiguous.
-  float flex = 1.0f;
-  if (a.x_scale) flex *= *a.x_scale;
-  if (a.w_scale) flex *= *a.w_scale;
-  float bias[NF];
-#pragma unroll
-  for (int f = 0; f < NF; ++f)
-    bias[f] = (a.bias && col0 + f < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col0 + f)
-                                       : 0.f;
-  constexpr int NO = ACT == TAMD_ACT_SWIGLU ? NF / 2 : NF;  // outputs per lane per row
-  constexpr int OUT_COLS = 128 * NO;                        // output columns of the tile
-  const int n_out = ACT == TAMD_ACT_SWIGLU ? N / 2 : N;
-  const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
-  const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
-  const bool has_limit = a.act_has_limit != 0;
-  const bool staged = a.y_dtype != TAMD_F32;
-  uint16_t *ob = (uint16_t *)lds;  // [rows][OUT_COLS]
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < NFR; ++i) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
-      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
-      const float beta = a.betas ? a.betas[erow] : 1.0f;
-      const float gamma = a.gammas ? a.gammas[erow] : 1.0f;
-      float v[NF];
-#pragma unroll
-      for (int f = 0; f < NF; ++f) v[f] = (acc[i][f][j] * flex + bias[f] * beta) * a.out_alpha;
-      float o[NO];
-      if constexpr (ACT == TAMD_ACT_SWIGLU) {
-        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit) * gamma;
-      } else {
-#pragma unroll
-        for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
-      }
-      if (staged) {
-        uint16_t *dstl = ob + r * OUT_COLS + wave * 32 * NO + c32 * NO;
-        if constexpr (NO == 2) {
-          uint32_t w2 = a.y_dtype == TAMD_BF16 ? (f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[NO - 1]) << 16))
-                                               : (f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[NO - 1]) << 16));
-          *(uint32_t *)dstl = w2;
-        } else {
-          *dstl = (uint16_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(o[0]) : f32_to_f16_bits(o[0]));
-        }
-      } else if (r < t.rows) {
-        int64_t dst = t.start_m + t.off_m + r;
-        if (a.scatter_indx) dst = a.scatter_indx[dst];
-        if (dst >= 0) {
-          const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
-#pragma unroll
-          for (int p = 0; p < NO; ++p)
-            if (out_col0 + p < n_out) ((float *)a.y)[base + out_col0 + p] = o[p];
-        }
-      }
-    }
-  }
-  if (staged) {
-    __syncthreads();
-    constexpr int CPR = OUT_COLS / 8;  // 16-byte chunks per tile row
-    const int n_chunks = t.rows * CPR;
-    for (int id = tid; id < n_chunks; id += 256) {
-      const int r = id / CPR, c = (id - r * CPR) * 8;
-      int64_t dst = t.start_m + t.off_m + r;
-      if (a.scatter_indx) dst = a.scatter_indx[dst];
-      if (dst < 0) continue;
-      const int gcol = tile_out0 + c;
-      if (gcol >= n_out) continue;
-      uint16_t *yp = (uint16_t *)a.y + (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol;
-      const uint16_t *sp = ob + r * OUT_COLS + c;
-      if (gcol + 8 <= n_out && ((uintptr_t)yp & 15) == 0) {
-        *(uint4 *)yp = *(const uint4 *)sp;
-      } else {
-        for (int e = 0; e < 8 && gcol + e < n_out; ++e) yp[e] = sp[e];
-      }
-    }
-  }
-}
-
-// BM: block size of the ragged schedule the kernel consumes (16..128).
-template <int XDT, int BM, int ACT, bool SC_LDS>
-__global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
-  constexpr int MF = BM <= 32 ? 1 : (BM == 128 ? 5 : BM / 32);  // 32-row fragments (128 + 32 absorbed)
-  constexpr int LDS_ROWS = 32 * MF;
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  Tile t;
-  if (!locate_tile<BM>(a, grid_n, grid_total, t)) return;
-  const int nfr = (t.rows + 31) / 32;  // active row fragments (workgroup uniform)
-#define TAMD_CASE(n)                                                           \
-  case n:                                                                      \
-    if constexpr (n <= MF) run_tile<XDT, n, LDS_ROWS, ACT, SC_LDS>(a, t, lds); \
-    break;
-  switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) TAMD_CASE(5) }
-#undef TAMD_CASE
-}
-
-template <int XDT, int BM, int ACT>
-int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int MF = BM <= 32 ? 1 : (BM == 128 ? 5 : BM / 32);
-  constexpr int LDS_ROWS = 32 * MF;
-  constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES;
-  constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
-  int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
-  int64_t total = (int64_t)grid_m * grid_n;
-  if (total <= 0) return 0;
-  int64_t launch = ((total + 7) / 8) * 8;
-  if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-  // scales of a tile are staged in LDS when they are dense ([N][K/32]) and two workgroups still fit a CU
-  const int64_t G = a.K / 32;
-  const int64_t sc_bytes = (BLOCK_N * G + 15) / 16 * 16;
-  const bool dense_sc = a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
-                        aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0;
-  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;
-  size_t lds_bytes = PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
-  if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;
-  auto kern = sc_in_lds ? mm_x16_mxfp4_kernel<XDT, BM, ACT, true> : mm_x16_mxfp4_kernel<XDT, BM, ACT, false>;
-  // raising the dynamic LDS limit is idempotent, so doing it on every launch keeps the entry point stateless
-  hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e != hipSuccess) return (int)e;
-  kern<<<dim3((unsigned)launch), 256, lds_bytes, st>>>(a, grid_n, total);
-  return launch_status();
-}
-
-template <int XDT, int BM>
-int launch_x16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  if (a.activation == TAMD_ACT_SWIGLU) return launch_x16_act<XDT, BM, TAMD_ACT_SWIGLU>(a, grid_m, st);
-  return launch_x16_act<XDT, BM, TAMD_ACT_NONE>(a, grid_m, st);
-}
-
-template <int XDT>
-int dispatch_x16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
-  switch (block_m) {
-    case 16: return launch_x16<XDT, 16>(a, grid_m, st);
-    case 32: return launch_x16<XDT, 32>(a, grid_m, st);
-    case 64: return launch_x16<XDT, 64>(a, grid_m, st);
-    case 128: return launch_x16<XDT, 128>(a, grid_m, st);
-    default: return TAMD_E_UNSUPPORTED;
-  }
-}
-
+int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int dispatch_mm_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int dispatch_mm_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 }  // namespace tamd
 
 using namespace tamd;
@@ -479,16 +26,18 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
   if (ragged && (!a.slice_sizes || !a.slice_offs || a.grid_m < 0)) return TAMD_E_INVALID;
   hipStream_t st = (hipStream_t)stream;
 
-  if (a.w_dtype == TAMD_MXFP4 && (a.x_dtype == TAMD_BF16 || a.x_dtype == TAMD_F16)) {
+  const bool x8 = a.x_dtype == TAMD_FP8_E4M3;
+  if (a.w_dtype == TAMD_MXFP4 && (a.x_dtype == TAMD_BF16 || a.x_dtype == TAMD_F16 || x8)) {
+    const int esz = x8 ? 1 : 2;
     if (!a.w_mx_scale) return TAMD_E_INVALID;
     if (a.K % 32 != 0) return TAMD_E_INVALID;
     // weights / scales must be contiguous along K ("column-major" mxfp weights)
     if (a.w_stride_k != 1 || a.w_mx_stride_k != 1) return TAMD_E_UNSUPPORTED;
     if (!aligned(a.w, 16) || a.w_stride_n % 16 != 0 || a.w_stride_e % 16 != 0) return TAMD_E_ALIGNMENT;
-    if (!aligned(a.x, 16) || (a.x_stride_m * 2) % 16 != 0 || (a.x_stride_z * 2) % 16 != 0) return TAMD_E_ALIGNMENT;
+    if (!aligned(a.x, 16) || (a.x_stride_m * esz) % 16 != 0 || (a.x_stride_z * esz) % 16 != 0) return TAMD_E_ALIGNMENT;
     // 32-bit buffer offsets: one batch of activations and one expert's weights must each span < 2 GiB
     const int64_t x_rows = a.x_rows > 0 ? a.x_rows : a.M;
-    if (x_rows * a.x_stride_m * 2 >= (int64_t)0x7FFFFF00 || (int64_t)a.N * a.w_stride_n >= (int64_t)0x7FFFFF00 ||
+    if (x_rows * a.x_stride_m * esz >= (int64_t)0x7FFFFF00 || (int64_t)a.N * a.w_stride_n >= (int64_t)0x7FFFFF00 ||
         (int64_t)a.N * a.w_mx_stride_n >= (int64_t)0x7FFFFF00)
       return TAMD_E_UNSUPPORTED;
     int block_m, grid_m;
@@ -499,8 +48,9 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
       block_m = a.force_variant ? a.force_variant : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128);
       grid_m = ((a.M + block_m - 1) / block_m) * a.n_experts;
     }
-    if (a.x_dtype == TAMD_BF16) return dispatch_x16<TAMD_BF16>(a, block_m, grid_m, st);
-    return dispatch_x16<TAMD_F16>(a, block_m, grid_m, st);
+    if (a.x_dtype == TAMD_BF16) return dispatch_mm_bf16(a, block_m, grid_m, st);
+    if (a.x_dtype == TAMD_F16) return dispatch_mm_f16(a, block_m, grid_m, st);
+    return dispatch_mm_fp8e4m3(a, block_m, grid_m, st);
   }
   return TAMD_E_UNSUPPORTED;
 }

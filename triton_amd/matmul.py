@@ -81,7 +81,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     """
     Y[dst(r), :] = act((X[src(r), :] @ W[e]) + bias[e] * betas[r]) * gammas[r]   for the rows r of every slice e
 
-    a: [M, K] activations (bf16 / fp16), or [B, M, K] batched.
+    a: [M, K] activations (bf16 / fp16, or float8_e4m3fn with flex_ctx.lhs_data.scale), or [B, M, K] batched.
     b: [E, K, N] weights; MXFP4 weights are uint8 with two codes per byte along K
        (storage [E, K/2, N] with unit stride along K) and precision_config.b_mx_scale
        holds their e8m0 scales [E, K/32, N].
@@ -145,6 +145,9 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
     out_dtype = precision_config.out_dtype or a.dtype
+    if out_dtype.itemsize == 1:
+        raise NotImplementedError("fp8 outputs need flexpoint output scaling, which is not built: "
+                                  "set precision_config.out_dtype to bfloat16 / float16 / float32")
     rows_out = M
     if gather_indx is not None:
         rows_out = gather_indx.shape[0]
