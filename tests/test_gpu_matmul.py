@@ -254,3 +254,60 @@ def test_moe_down_projection_and_combine_small(device):
     z, _ = reduce(y.view(T, k, N), dim=1)
     z_ref = MR.reduce_ref(y.cpu().view(T, k, N), 1)
     assert torch.equal(z.cpu(), z_ref)  # fixed summation order: the combine is bit-exact given y
+
+
+# ---------------------------------------------------------------------------- decode: weight-streaming kernel
+
+
+@pytest.mark.parametrize("K", [64, 320, 1024, 2048, 2880, 4096])
+@pytest.mark.parametrize("act,bias_dtype,xdtype", [(True, torch.bfloat16, torch.bfloat16), (False, torch.float32, torch.bfloat16),
+                                                   (True, torch.float16, torch.float16)])
+def test_decode_row_blocks_of_16(K, act, bias_dtype, xdtype, device):
+    """Few rows per expert, N a multiple of 16, K dense per column: the streaming kernel (split-K over the
+    waves, linear weight images) against the oracle; gather, scatter with dropped rows, gate weights."""
+    torch.manual_seed(K)
+    E, N = 7, 608
+    sizes = torch.tensor([3, 0, 1, 16, 5, 21, 2], dtype=torch.int32)  # 21 rows: two row blocks for one expert
+    M = int(sizes.sum())
+    x = torch.randn(M + 5, K).to(xdtype)
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N).to(bias_dtype)
+    v, s, rv, rs = quantize_w(w, device)
+    gather = torch.randint(0, M + 5, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::7] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    out_init = torch.zeros((M, N // 2 if act else N), dtype=xdtype, device=device)
+    with scoped_opt_flags_constraints({"block_m": 16}):
+        out = matmul(x.to(device), v, bias.to(device), md, gather_indx=gather.to(device), scatter_indx=scatter.to(device),
+                     precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0) if act else None,
+                     c=out_init)
+    ref = MR.matmul_ref(x, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs,
+                        gammas=gammas, fused_swiglu=(1.702, 7.0) if act else None)
+    check(out, ref)
+
+
+def test_decode_shape_of_the_baseline(device):
+    """Config 4 at reduced expert count: T=64 tokens, top-4 of 16 experts, K=2880, N=5760, bias + SwiGLU."""
+    torch.manual_seed(0)
+    T, E, k, H, N = 64, 16, 4, 2880, 5760
+    logits = torch.randn(T, E)
+    x = torch.randn(T, H).to(torch.bfloat16)
+    bias = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
+    v = torch.empty((E, H // 2, N), dtype=torch.uint8, device=device).transpose(1, 2).contiguous().transpose(1, 2)
+    s = torch.empty((E, H // 32, N), dtype=torch.uint8, device=device).transpose(1, 2).contiguous().transpose(1, 2)
+    rv, rs = torch.empty_like(v, device="cpu"), torch.empty_like(s, device="cpu")
+    for e in range(E):
+        ve, se, rve, rse = quantize_w(torch.randn(1, H, N) * 0.02, device)
+        v[e].copy_(ve[0]), s[e].copy_(se[0]), rv[e].copy_(rve[0]), rs[e].copy_(rse[0])
+    r = routing(logits.to(device), k)
+    rr = RR.routing_ref(logits, k)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    with scoped_opt_flags_constraints({"block_m": 16}):
+        out = matmul(x.to(device), v, bias.to(device), r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc,
+                     fused_activation=swiglu_act(1.702, 7.0))
+    ref = MR.matmul_ref(x, rv, bias, slice_sizes=rr["col_sum"], gather_indx=rr["gather_indx"], b_mx_scale=rs,
+                        fused_swiglu=(1.702, 7.0))
+    check(out, ref)

@@ -1,8 +1,13 @@
-// Instantiates the grouped matmul kernels of moe_matmul_impl.h for one activation type.
-#include "moe_matmul_impl.h"
+// Instantiates the grouped matmul kernels for one activation type: the streaming kernel for row blocks of
+// 16 (moe_matmul_stream.h) and the tiled kernel for everything else (moe_matmul_impl.h).
+#include "moe_matmul_stream.h"
 
 namespace tamd {
 int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  if (block_m == 16 && stream16_applicable(a)) {
+    if (a.activation == TAMD_ACT_SWIGLU) return launch_stream16<TAMD_BF16, TAMD_ACT_SWIGLU>(a, grid_m, st);
+    return launch_stream16<TAMD_BF16, TAMD_ACT_NONE>(a, grid_m, st);
+  }
   return dispatch_x16<TAMD_BF16>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

@@ -150,10 +150,12 @@ TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid
 // 128-bit global -> LDS copy that bypasses registers (buffer_load ... lds).  The LDS destination of
 // lane L is lds_addr + 16*L; out-of-range offsets (>= num_records of the descriptor) deliver zeros.
 // Issued through inline asm so that the compiler does not serialise later LDS reads behind it; the
-// kernel waits for these copies itself (wait_dma) before the barrier that publishes a stage.
+// kernel waits for these copies itself (wait_dma) before the barrier that publishes a stage.  The
+// five wait states cover an SGPR operand written by a v_readfirstlane just before the block (the
+// compiler's hazard recognizer does not look inside inline asm) and the write of M0.
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 TAMD_DEVICE void dma16(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
                  "s"(__builtin_amdgcn_readfirstlane(soff))

@@ -1,0 +1,386 @@
+// Weight-streaming grouped matmul for row blocks of at most 16 rows (decode): 16-bit activations x
+// MXFP4 weights.  Same arithmetic as the tiled kernel of moe_matmul_impl.h; the design goal here is
+// HBM bandwidth, since with a handful of rows per expert every weight byte is used exactly once.
+//
+// Measured on this part: reading 128 bytes of every column per K step (columns 1440 bytes apart)
+// tops out near 3.4 TB/s, a linear read reaches 6.2 TB/s.  So the kernel reads the weights in
+// memory order:
+//   * a unit of work is (row block, group of 16 consecutive columns).  With K contiguous per column
+//     the 16 columns are one contiguous run of 16*K/2 bytes (plus 16*K/32 scale bytes);
+//   * one workgroup (4 waves) per CU walks a contiguous range of units, cut from the number of real
+//     row blocks read on the device (block_offs[n_experts]), so consecutive units continue the same
+//     linear stream and the padding of the block schedule costs nothing;
+//   * the runs go HBM -> LDS by DMA (buffer_load ... lds) as they lie in memory, through a ring of
+//     stages filled several units ahead (about 100 KB in flight per CU); every per-unit operand,
+//     bias included, travels in that DMA stream so that no other load ever drains it;
+//   * the K range is split over the four waves (split-K inside the workgroup): wave w keeps its
+//     quarter of the up-to-16 activation rows in registers for as long as the row block lasts, so
+//     activations never occupy LDS; partial 16x16 results are summed through LDS one unit later,
+//     by the threads that also apply bias / activation / gate weight and store.
+//   * v_mfma_f32_16x16x32: lane (c = lane%16, g = lane/16) is row c of A and column c of B; in super
+//     step j of wave w it owns e8m0 group 4*SS*w + 4j + g (32 K), consumed 8 K at a time by 4 MFMAs.
+#pragma once
+#include "moe_matmul_impl.h"
+
+#ifndef TAMD_STREAM_WGS_PER_CU
+#define TAMD_STREAM_WGS_PER_CU 1
+#endif
+
+namespace tamd {
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int XDT>
+struct Mma16;
+template <>
+struct Mma16<TAMD_BF16> {
+  static TAMD_DEVICE f32x4_t mma(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma16<TAMD_F16> {
+  static TAMD_DEVICE f32x4_t mma(f16x8_t a, f16x8_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 2- and 4-byte global -> LDS copies: lane L's value lands (zero-extended) in the dword at
+// lds_addr + 4*L; out-of-range offsets deliver zero.  The five wait states before the load cover an
+// SGPR operand that a v_readfirstlane wrote just before the asm block (the compiler's hazard
+// recognizer does not look inside inline asm) as well as the write of M0.
+TAMD_DEVICE void dma2(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_ushort %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+TAMD_DEVICE void dma4(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding).
+template <int N>
+TAMD_DEVICE void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+  asm volatile("" ::: "memory");
+}
+
+// 16-byte copies with an instruction offset: OFF is added to the global offset and to the LDS address
+// alike, so one M0 value serves up to four consecutive 1 KB pieces of a linear image.
+// SETM0: also loads M0 with lds_addr first (with the wait states an SGPR operand written by a
+// preceding v_readfirstlane needs; pieces that follow reuse the same registers).
+template <int OFF, bool SETM0>
+TAMD_DEVICE void dma16_at(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  if constexpr (SETM0)
+    asm volatile("s_mov_b32 m0, %4\n\ts_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds"
+                 :
+                 : "v"(voff), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(soff)), "n"(OFF),
+                   "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+                 : "memory", "m0");
+  else
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds"
+                 :
+                 : "v"(voff), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(soff)), "n"(OFF)
+                 : "memory");
+}
+
+template <int SS, int RING_>
+struct StreamShape {
+  static constexpr int CODE_BYTES = 4 * SS * 1024;  // image of 16 columns' codes, padded to whole 1 KB copies
+  static constexpr int SC_BYTES = 2048;             // image of their scales (16 * K/32 <= 2048 bytes)
+  static constexpr int BIAS_BYTES = 512;            // 16 bias values, one dword each; second half takes wave 3's empty copy
+  static constexpr int STAGE = CODE_BYTES + SC_BYTES + BIAS_BYTES;
+  static constexpr int RED_BYTES = 2 * 4 * 1024;    // partial sums: 2 buffers x 4 waves x 16x16 floats
+  static constexpr int RING = RING_;
+  static constexpr int DMA_PER_STAGE = SS + 1;      // per wave
+  static constexpr int LDS = RING * STAGE + RED_BYTES;
+  static_assert(RING >= 2 && (RING - 1) * DMA_PER_STAGE < 64, "ring does not fit the vmcnt counter");
+};
+
+// SS: super steps (4 e8m0 groups = 128 K each) per wave; covers K <= 512 * SS.  N is a multiple of 16.
+template <int XDT, int ACT, int SS, int RING, int WGS_PER_CU>
+__global__ __launch_bounds__(256, WGS_PER_CU) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
+  typedef Mma<XDT> M;
+  typedef typename M::frag_t frag_t;
+  typedef StreamShape<SS, RING> S;
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr uint32_t kOob = 0x7FFFFFFFu;
+  constexpr bool SW = ACT == TAMD_ACT_SWIGLU;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+  const int c16 = lane % 16, g = lane / 16;
+  const int er = tid / 16, ec = tid % 16;  // epilogue thread -> (row, column) of the 16x16 result
+  const int K = a.K, N = a.N, G = K / 32;
+  const uint32_t col_bytes = (uint32_t)(K / 2);
+
+  // ---- this workgroup's range of units
+  const int n_blocks = a.block_schedule ? a.block_offs[a.n_experts] : dense_blocks;
+  const int64_t total = (int64_t)n_blocks * n_cg;
+  const int64_t first = (int64_t)blockIdx.x * total / gridDim.x;
+  const int64_t last = (int64_t)(blockIdx.x + 1) * total / gridDim.x;
+  if (first >= last) return;
+  const int total_stages = (int)(last - first);
+  const int blk0 = (int)(first / n_cg), cg0 = (int)(first - (int64_t)blk0 * n_cg);
+
+  struct Block {  // a row block of at most 16 rows
+    int expert, z, row0, rows;
+  };
+  auto get_block = [&](int blk, Block &b) {
+    b.z = 0;
+    int slice_rows, off_m;
+    if (a.block_schedule) {
+      const int sched = a.block_schedule[blk];
+      if (sched == -1) {  // cannot happen below block_offs[n_experts]; an empty block keeps the ring in step
+        b.expert = 0, b.row0 = 0, b.rows = 0;
+        return;
+      }
+      b.expert = sched & 0xFFFF;
+      slice_rows = a.slice_sizes[b.expert];
+      off_m = (sched >> 16) * 16;
+      b.row0 = a.slice_offs[b.expert] + off_m;
+    } else {
+      const int bm = (a.M + 15) / 16;
+      const int z = blk / bm;
+      b.expert = z, b.z = z;
+      slice_rows = a.M;
+      off_m = (blk - z * bm) * 16;
+      b.row0 = off_m;
+    }
+    const int left = slice_rows - off_m;
+    b.rows = left > 16 ? 16 : (left < 0 ? 0 : left);
+  };
+
+  // live descriptors, and empty ones (no records: every lane out of range) for copies past the end
+  const v4i_t rw = make_rsrc(a.w, kOob), rs = make_rsrc(a.w_mx_scale, kOob), rb = make_rsrc(a.bias, kOob);
+  const v4i_t rw0 = make_rsrc(a.w, 0), rs0 = make_rsrc(a.w_mx_scale, 0), rb0 = make_rsrc(a.bias, 0);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  float *red = (float *)(lds + S::RING * S::STAGE);
+  const int bias_esz = a.bias_dtype == TAMD_F32 ? 4 : 2;
+
+  // ---- issue side.  Per-lane source offsets never change: a unit's codes, scales and bias are linear
+  // images.  Past the end of the range the same number of copies is issued through the empty
+  // descriptors, so that the count of outstanding copies per stage stays the same.
+  uint32_t w_voff[SS];
+#pragma unroll
+  for (int i = 0; i < SS; ++i) {
+    const uint32_t lin = (uint32_t)(wave * SS + i) * 1024u + lane * 16u;
+    w_voff[i] = lin < 16u * col_bytes ? (uint32_t)(wave * SS) * 1024u + lane * 16u : kOob;  // piece i adds i*1024 itself
+  }
+  uint32_t x_voff;  // the extra copy: scales (waves 0, 1), bias (wave 2), nothing (wave 3)
+  if (wave < 2) x_voff = (uint32_t)wave * 1024u + lane * 16u < (uint32_t)(16 * G) ? (uint32_t)wave * 1024u + lane * 16u : kOob;
+  else x_voff = (wave == 2 && a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
+  int i_blk = blk0 - 1, i_cg = cg0, i_left = total_stages;
+  uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0;
+  auto issue = [&](int slot) {
+    const bool live = i_left > 0;
+    if (live && (i_blk < blk0 || i_cg == n_cg)) {
+      if (i_cg == n_cg) i_cg = 0;
+      ++i_blk;
+      Block b;
+      get_block(i_blk, b);
+      const int e = __builtin_amdgcn_readfirstlane(b.expert);  // keeps the running offsets in scalar registers
+      i_wbase = (uint32_t)((int64_t)e * a.w_stride_e) + (uint32_t)i_cg * 16u * col_bytes;
+      i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e) + (uint32_t)(i_cg * 16 * G);
+      i_bbase = (uint32_t)(((int64_t)e * a.bias_stride_e + i_cg * 16) * bias_esz);
+    }
+    const uint32_t sb = lds_base + slot * S::STAGE;
+    const v4i_t dw = live ? rw : rw0;
+#pragma unroll
+    for (int i = 0; i < SS; ++i) {
+      const uint32_t m0v = sb + (wave * SS + i / 4 * 4) * 1024;
+      const uint32_t so = i_wbase + (uint32_t)(i / 4) * 4096u;
+      if (i % 4 == 0) dma16_at<0, true>(dw, m0v, w_voff[i], so);
+      if (i % 4 == 1) dma16_at<1024, false>(dw, m0v, w_voff[i], so);
+      if (i % 4 == 2) dma16_at<2048, false>(dw, m0v, w_voff[i], so);
+      if (i % 4 == 3) dma16_at<3072, false>(dw, m0v, w_voff[i], so);
+    }
+    if (wave < 2) {
+      dma16(live ? rs : rs0, sb + S::CODE_BYTES + wave * 1024, x_voff, i_sbase);
+    } else {
+      const uint32_t dst = sb + S::CODE_BYTES + S::SC_BYTES + (wave - 2) * 256;  // an empty copy writes zeros
+      if (bias_esz == 4) dma4(live ? rb : rb0, dst, x_voff, i_bbase);
+      else dma2(live ? rb : rb0, dst, x_voff, i_bbase);
+    }
+    ++i_cg, --i_left;
+    i_wbase += 16u * col_bytes, i_sbase += (uint32_t)(16 * G), i_bbase += (uint32_t)(16 * bias_esz);
+  };
+
+  // ---- compute side state: the row block whose activations sit in registers
+  frag_t areg[SS * 4];
+  int c_blk = blk0 - 1, c_cg = cg0;
+  Block cb;
+  float row_beta = 1.f, row_gamma = 1.f;
+  int64_t row_dst = -1;
+  const int kb = 4 * SS * wave;  // first e8m0 group of this wave's K slice
+  auto load_block = [&](int blk) {
+    get_block(blk, cb);
+    int rc = c16 < cb.rows ? c16 : cb.rows - 1;
+    rc = cb.row0 + (rc < 0 ? 0 : rc);
+    const int64_t src = a.gather_indx ? (int64_t)a.gather_indx[rc] : (int64_t)rc;
+    const uint16_t *xr = (const uint16_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+#pragma unroll
+    for (int j = 0; j < SS; ++j) {
+      const int kg = kb + 4 * j + g;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (kg < G && cb.rows > 0) v = *(const uint4 *)(xr + 32 * kg + 8 * u);
+        areg[j * 4 + u] = __builtin_bit_cast(frag_t, v);
+      }
+    }
+    const bool rv = er < cb.rows;
+    const int erow = cb.row0 + (rv ? er : 0);
+    row_beta = (a.betas && rv) ? a.betas[erow] : 1.0f;
+    row_gamma = (a.gammas && rv) ? a.gammas[erow] : 1.0f;
+    row_dst = rv ? (a.scatter_indx ? (int64_t)a.scatter_indx[erow] : (int64_t)erow) : -1;
+    row_dst = row_dst < 0 ? -1 : (int64_t)cb.z * a.y_stride_z + row_dst * a.y_stride_m;
+  };
+  // per-lane LDS offsets of this wave's K slice inside a stage (beyond K: group 0 with scale 1.0 --
+  // the activations there are zero, the weight operand only has to stay finite)
+  uint32_t b_loff[SS], s_loff[SS];
+  bool kvalid[SS];
+#pragma unroll
+  for (int j = 0; j < SS; ++j) {
+    const int kg = kb + 4 * j + g;
+    kvalid[j] = kg < G;
+    b_loff[j] = (uint32_t)c16 * col_bytes + (kvalid[j] ? kg : 0) * 16;
+    s_loff[j] = (uint32_t)(S::CODE_BYTES + c16 * G + (kvalid[j] ? kg : 0));
+  }
+
+  float flex = 1.0f;
+  if (a.x_scale) flex *= *a.x_scale;
+  if (a.w_scale) flex *= *a.w_scale;
+  const bool has_limit = a.act_has_limit != 0;
+  const int n_out = SW ? N / 2 : N;
+  const int red_idx = ((er >> 2) * 16 + ec) * 4 + (er & 3);
+
+  // what the deferred epilogue of the previous unit needs
+  float p_bias = 0.f, p_beta = 1.f, p_gamma = 1.f;
+  int64_t p_dst = -1;
+  int p_col0 = 0;
+  auto epilogue = [&](int buf) {
+    const float *rbuf = red + buf * 1024 + red_idx;
+    const float sum = (rbuf[0] + rbuf[256]) + (rbuf[512] + rbuf[768]);
+    float v = (sum * flex + p_bias * p_beta) * a.out_alpha;
+    int col = p_col0 + ec;
+    bool store = p_dst >= 0;
+    if constexpr (SW) {
+      const float other = __shfl_xor(v, 1);
+      v = swiglu_fast(v, other, a.act_alpha, a.act_limit, has_limit);
+      store = store && (ec & 1) == 0;
+      col >>= 1;
+    }
+    v *= p_gamma;
+    if (store && col < n_out) {
+      const int64_t at = p_dst + col;
+      if (a.y_dtype == TAMD_F32) ((float *)a.y)[at] = v;
+      else ((uint16_t *)a.y)[at] = (uint16_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+    }
+  };
+
+  // ---- the ring: stage s lives in slot s % RING and is requested RING - 1 stages ahead
+  int i_slot = 0;
+#pragma unroll 1
+  for (int s = 0; s < S::RING - 1; ++s) {
+    issue(i_slot);
+    i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
+  }
+  int slot = 0;
+#pragma unroll 1
+  for (int s = 0; s < total_stages; ++s) {
+    // copies complete in order: once at most RING - 2 stages' worth are outstanding, stage s has landed
+    wait_vmcnt<(S::RING - 2) * S::DMA_PER_STAGE>();
+    __syncthreads();  // stage s and the partial sums of stage s - 1 are visible; slot (s - 1) % RING is free
+    issue(i_slot);
+    i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
+    if (s > 0) epilogue((s - 1) & 1);
+    if (c_blk < blk0 || c_cg == n_cg) {
+      if (c_cg == n_cg) c_cg = 0;
+      load_block(++c_blk);
+    }
+
+    const uint8_t *img = lds + slot * S::STAGE;
+    f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+#pragma unroll
+    for (int j = 0; j < SS; ++j) {
+      const uint4 r = *(const uint4 *)(img + b_loff[j]);
+      const uint32_t sbyte = kvalid[j] ? (uint32_t)img[s_loff[j]] : 127u;
+      const float sc = bits_to_f32(sbyte << 23);
+      acc0 = Mma16<XDT>::mma(areg[j * 4 + 0], M::expand(r.x, sc), acc0);
+      acc1 = Mma16<XDT>::mma(areg[j * 4 + 1], M::expand(r.y, sc), acc1);
+      acc0 = Mma16<XDT>::mma(areg[j * 4 + 2], M::expand(r.z, sc), acc0);
+      acc1 = Mma16<XDT>::mma(areg[j * 4 + 3], M::expand(r.w, sc), acc1);
+    }
+    *(f32x4_t *)(red + (s & 1) * 1024 + wave * 256 + lane * 4) = acc0 + acc1;
+
+    // carry this unit's epilogue operands to the next iteration
+    const uint32_t braw = *(const uint32_t *)(img + S::CODE_BYTES + S::SC_BYTES + ec * 4);
+    p_bias = a.bias == nullptr ? 0.f
+                               : (a.bias_dtype == TAMD_F32 ? bits_to_f32(braw)
+                                                           : (a.bias_dtype == TAMD_BF16 ? bits_to_f32(braw << 16)
+                                                                                        : f16_bits_to_f32((uint16_t)braw)));
+    p_beta = row_beta, p_gamma = row_gamma, p_dst = row_dst;
+    p_col0 = c_cg * 16;
+    ++c_cg;
+    slot = slot + 1 == S::RING ? 0 : slot + 1;
+  }
+  __syncthreads();
+  epilogue((total_stages - 1) & 1);
+  wait_vmcnt<0>();  // the empty copies issued past the end still write (zeros) to LDS
+}
+
+// Whether the streaming kernel covers the problem: K contiguous and dense per column for codes and
+// scales, 16-byte aligned column groups, N a multiple of 16, K <= 4096, whole tensors addressable
+// with 32-bit offsets.
+inline bool stream16_applicable(const tamd_matmul_args &a) {
+  const int64_t lim = 0x7FFFFF00;
+  const int64_t G = a.K / 32;
+  if (a.K > 4096 || a.K % 32 != 0) return false;
+  if (a.w_stride_k != 1 || a.w_stride_n != a.K / 2 || a.w_mx_stride_k != 1 || a.w_mx_stride_n != G) return false;
+  if (!aligned(a.w, 16) || a.w_stride_e % 16 != 0 || !aligned(a.w_mx_scale, 16) || a.w_mx_stride_e % 16 != 0) return false;
+  if ((int64_t)a.n_experts * a.w_stride_e + (int64_t)a.N * a.w_stride_n >= lim) return false;
+  if ((int64_t)a.n_experts * a.w_mx_stride_e + (int64_t)a.N * G >= lim) return false;
+  if (a.bias && ((int64_t)a.n_experts * a.bias_stride_e + a.N) * 4 >= lim) return false;
+  if (a.bias && !aligned(a.bias, a.bias_dtype == TAMD_F32 ? 4 : 2)) return false;
+  if (a.N % 16 != 0) return false;  // whole 16-column groups only (their scale run is then a multiple of 16 bytes)
+  if (a.block_schedule && !a.block_offs) return false;
+  return true;
+}
+
+template <int XDT, int ACT, int SS>
+int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  constexpr int WGS_PER_CU = TAMD_STREAM_WGS_PER_CU;
+  constexpr int RING_FIT = ((WGS_PER_CU == 1 ? 156 : 80) * 1024 - 8192) / (4 * SS * 1024 + 2048 + 512);
+  constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
+  const int n_cg = (a.N + 15) / 16;
+  const int64_t upper = (int64_t)grid_m * n_cg;
+  if (upper <= 0) return 0;
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  const int wgs = (int)(upper < cus * WGS_PER_CU ? upper : cus * WGS_PER_CU);
+  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, WGS_PER_CU>;
+  e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  kern<<<dim3((unsigned)wgs), 256, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
+  return launch_status();
+}
+
+template <int XDT, int ACT>
+int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  const int ss = (a.K / 32 + 15) / 16;  // super steps per wave
+  if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2>(a, grid_m, st);
+  if (ss <= 4) return launch_stream16_ss<XDT, ACT, 4>(a, grid_m, st);
+  if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6>(a, grid_m, st);
+  return launch_stream16_ss<XDT, ACT, 8>(a, grid_m, st);
+}
+
+}  // namespace tamd
