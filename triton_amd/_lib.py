@@ -10,7 +10,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtriton_amd.so")
+LIB_PATH = os.environ.get("TAMD_LIB") or os.path.join(_HERE, "libtriton_amd.so")  # TAMD_LIB: another build of the same ABI
 
 # element type codes (include/triton_amd.h)
 F32, F16, BF16, FP8_E4M3, FP8_E5M2, MXFP4 = 0, 1, 2, 3, 4, 5

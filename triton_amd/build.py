@@ -18,8 +18,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 
+EXTRA = os.environ.get("TAMD_EXTRA_HIPCC_FLAGS", "").split()  # e.g. -DTAMD_STREAM_WGS_PER_CU=1 for experiments
+
+
 def _compile(src, obj):
-    cmd = [HIPCC, *FLAGS, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")

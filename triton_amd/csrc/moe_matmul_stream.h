@@ -7,23 +7,24 @@
 // memory order:
 //   * a unit of work is (row block, group of 16 consecutive columns).  With K contiguous per column
 //     the 16 columns are one contiguous run of 16*K/2 bytes (plus 16*K/32 scale bytes);
-//   * one workgroup (4 waves) per CU walks a contiguous range of units, cut from the number of real
-//     row blocks read on the device (block_offs[n_experts]), so consecutive units continue the same
-//     linear stream and the padding of the block schedule costs nothing;
-//   * the runs go HBM -> LDS by DMA (buffer_load ... lds) as they lie in memory, through a ring of
-//     stages filled several units ahead (about 100 KB in flight per CU); every per-unit operand,
-//     bias included, travels in that DMA stream so that no other load ever drains it;
-//   * the K range is split over the four waves (split-K inside the workgroup): wave w keeps its
-//     quarter of the up-to-16 activation rows in registers for as long as the row block lasts, so
-//     activations never occupy LDS; partial 16x16 results are summed through LDS one unit later,
-//     by the threads that also apply bias / activation / gate weight and store.
+//   * one workgroup per CU walks a contiguous range of units, cut from the number of real row blocks
+//     read on the device (block_offs[n_experts]), so consecutive units continue the same linear
+//     stream and the padding of the block schedule costs nothing;
+//   * two waves copy, four compute, two finish.  The copying waves send the runs HBM -> LDS by DMA
+//     (buffer_load ... lds) as they lie in memory, through a ring of stages filled several units
+//     ahead (about 100 KB in flight per CU); every per-unit operand, bias included, travels in that
+//     stream so that no other load ever drains it;
+//   * the K range is split over the four compute waves (split-K inside the workgroup): wave w keeps
+//     its quarter of the up-to-16 activation rows in registers for as long as the row block lasts,
+//     so activations never occupy LDS; partial 16x16 results go through LDS to the finishing waves,
+//     which apply bias / activation / gate weight and store one unit later;
 //   * v_mfma_f32_16x16x32: lane (c = lane%16, g = lane/16) is row c of A and column c of B; in super
 //     step j of wave w it owns e8m0 group 4*SS*w + 4j + g (32 K), consumed 8 K at a time by 4 MFMAs.
 #pragma once
 #include "moe_matmul_impl.h"
 
-#ifndef TAMD_STREAM_WGS_PER_CU
-#define TAMD_STREAM_WGS_PER_CU 1
+#ifndef TAMD_ABL
+#define TAMD_ABL 0  // timing experiments only: 1 = no epilogue, 2 = one super step, 4 = no wait for the copies
 #endif
 
 namespace tamd {
@@ -95,18 +96,23 @@ template <int SS, int RING_>
 struct StreamShape {
   static constexpr int CODE_BYTES = 4 * SS * 1024;  // image of 16 columns' codes, padded to whole 1 KB copies
   static constexpr int SC_BYTES = 2048;             // image of their scales (16 * K/32 <= 2048 bytes)
-  static constexpr int BIAS_BYTES = 512;            // 16 bias values, one dword each; second half takes wave 3's empty copy
+  static constexpr int BIAS_BYTES = 256;            // 16 bias values, one dword each
   static constexpr int STAGE = CODE_BYTES + SC_BYTES + BIAS_BYTES;
   static constexpr int RED_BYTES = 2 * 4 * 1024;    // partial sums: 2 buffers x 4 waves x 16x16 floats
   static constexpr int RING = RING_;
-  static constexpr int DMA_PER_STAGE = SS + 1;      // per wave
+  static constexpr int DMA_PER_STAGE = 2 * SS + 2;  // most copies one wave has per stage
   static constexpr int LDS = RING * STAGE + RED_BYTES;
   static_assert(RING >= 2 && (RING - 1) * DMA_PER_STAGE < 64, "ring does not fit the vmcnt counter");
 };
 
 // SS: super steps (4 e8m0 groups = 128 K each) per wave; covers K <= 512 * SS.  N is a multiple of 16.
-template <int XDT, int ACT, int SS, int RING, int WGS_PER_CU>
-__global__ __launch_bounds__(256, WGS_PER_CU) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
+//
+// 512 threads in three roles: waves 0-3 compute (LDS -> convert -> MFMA -> partial sums), waves 4-5
+// issue and await the copies, waves 6-7 finish and store the previous unit.  A wave that issues copies
+// stalls whenever the memory pipeline is full; with nothing else to do it refills the pipeline the
+// moment there is room, and the stalls never delay MFMA work or stores.
+template <int XDT, int ACT, int SS, int RING>
+__global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
   typedef StreamShape<SS, RING> S;
@@ -114,9 +120,8 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void mm_stream16_kernel(tamd_matmu
   constexpr uint32_t kOob = 0x7FFFFFFFu;
   constexpr bool SW = ACT == TAMD_ACT_SWIGLU;
   const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
-  const int c16 = lane % 16, g = lane / 16;
-  const int er = tid / 16, ec = tid % 16;  // epilogue thread -> (row, column) of the 16x16 result
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+  const int wave = wave8 & 3;  // index inside its group of four
   const int K = a.K, N = a.N, G = K / 32;
   const uint32_t col_bytes = (uint32_t)(K / 2);
 
@@ -156,184 +161,241 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void mm_stream16_kernel(tamd_matmu
     const int left = slice_rows - off_m;
     b.rows = left > 16 ? 16 : (left < 0 ? 0 : left);
   };
-
-  // live descriptors, and empty ones (no records: every lane out of range) for copies past the end
-  const v4i_t rw = make_rsrc(a.w, kOob), rs = make_rsrc(a.w_mx_scale, kOob), rb = make_rsrc(a.bias, kOob);
-  const v4i_t rw0 = make_rsrc(a.w, 0), rs0 = make_rsrc(a.w_mx_scale, 0), rb0 = make_rsrc(a.bias, 0);
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
   float *red = (float *)(lds + S::RING * S::STAGE);
-  const int bias_esz = a.bias_dtype == TAMD_F32 ? 4 : 2;
 
-  // ---- issue side.  Per-lane source offsets never change: a unit's codes, scales and bias are linear
-  // images.  Past the end of the range the same number of copies is issued through the empty
-  // descriptors, so that the count of outstanding copies per stage stays the same.
-  uint32_t w_voff[SS];
-#pragma unroll
-  for (int i = 0; i < SS; ++i) {
-    const uint32_t lin = (uint32_t)(wave * SS + i) * 1024u + lane * 16u;
-    w_voff[i] = lin < 16u * col_bytes ? (uint32_t)(wave * SS) * 1024u + lane * 16u : kOob;  // piece i adds i*1024 itself
-  }
-  uint32_t x_voff;  // the extra copy: scales (waves 0, 1), bias (wave 2), nothing (wave 3)
-  if (wave < 2) x_voff = (uint32_t)wave * 1024u + lane * 16u < (uint32_t)(16 * G) ? (uint32_t)wave * 1024u + lane * 16u : kOob;
-  else x_voff = (wave == 2 && a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
-  int i_blk = blk0 - 1, i_cg = cg0, i_left = total_stages;
-  uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0;
-  auto issue = [&](int slot) {
-    const bool live = i_left > 0;
-    if (live && (i_blk < blk0 || i_cg == n_cg)) {
-      if (i_cg == n_cg) i_cg = 0;
-      ++i_blk;
-      Block b;
-      get_block(i_blk, b);
-      const int e = __builtin_amdgcn_readfirstlane(b.expert);  // keeps the running offsets in scalar registers
-      i_wbase = (uint32_t)((int64_t)e * a.w_stride_e) + (uint32_t)i_cg * 16u * col_bytes;
-      i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e) + (uint32_t)(i_cg * 16 * G);
-      i_bbase = (uint32_t)(((int64_t)e * a.bias_stride_e + i_cg * 16) * bias_esz);
+  if (wave8 >= 6) {
+    // =========================================================================== finishing waves
+    // 128 threads: thread -> (row er, column pair pc) of the 16x16 result of a unit; they read the four
+    // partial sums one stage late, apply scale / bias / activation / gate weight and store.  These
+    // waves never issue copies, so their loads and stores do not interfere with the copy counters.
+    const int ft = tid - 384;
+    const int er = ft / 8, pc = ft % 8;
+    float flex = 1.0f;
+    if (a.x_scale) flex *= *a.x_scale;
+    if (a.w_scale) flex *= *a.w_scale;
+    const bool has_limit = a.act_has_limit != 0;
+    const int n_out = SW ? N / 2 : N;
+    const int red_idx = ((er >> 2) * 16 + 2 * pc) * 4 + (er & 3);  // column 2*pc; column 2*pc + 1 is 4 floats on
+    int c_blk = blk0 - 1, c_cg = cg0;
+    float row_beta = 1.f, row_gamma = 1.f, p_bias0 = 0.f, p_bias1 = 0.f, p_beta = 1.f, p_gamma = 1.f;
+    int64_t row_dst = -1, p_dst = -1;
+    int p_col0 = 0;
+    auto load_rows = [&](int blk) {
+      Block cb;
+      get_block(blk, cb);
+      const bool rv = er < cb.rows;
+      const int erow = cb.row0 + (rv ? er : 0);
+      row_beta = (a.betas && rv) ? a.betas[erow] : 1.0f;
+      row_gamma = (a.gammas && rv) ? a.gammas[erow] : 1.0f;
+      row_dst = rv ? (a.scatter_indx ? (int64_t)a.scatter_indx[erow] : (int64_t)erow) : -1;
+      row_dst = row_dst < 0 ? -1 : (int64_t)cb.z * a.y_stride_z + row_dst * a.y_stride_m;
+    };
+    auto to_f32 = [&](uint32_t raw) {
+      return a.bias == nullptr ? 0.f
+                               : (a.bias_dtype == TAMD_F32 ? bits_to_f32(raw)
+                                                           : (a.bias_dtype == TAMD_BF16 ? bits_to_f32(raw << 16)
+                                                                                        : f16_bits_to_f32((uint16_t)raw)));
+    };
+    auto to_16 = [&](float v) {
+      return (uint32_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v)) & 0xFFFFu;
+    };
+    auto finish = [&](int buf) {
+      const float *rbuf = red + buf * 1024 + red_idx;
+      const float s0 = (rbuf[0] + rbuf[256]) + (rbuf[512] + rbuf[768]);
+      const float s1 = (rbuf[4] + rbuf[260]) + (rbuf[516] + rbuf[772]);
+      const float v0 = (s0 * flex + p_bias0 * p_beta) * a.out_alpha;
+      const float v1 = (s1 * flex + p_bias1 * p_beta) * a.out_alpha;
+      if (p_dst < 0) return;
+      if constexpr (SW) {
+        const int col = (p_col0 >> 1) + pc;
+        if (col >= n_out) return;
+        const float o = swiglu_fast(v0, v1, a.act_alpha, a.act_limit, has_limit) * p_gamma;
+        if (a.y_dtype == TAMD_F32) ((float *)a.y)[p_dst + col] = o;
+        else ((uint16_t *)a.y)[p_dst + col] = (uint16_t)to_16(o);
+      } else {
+        const int col = p_col0 + 2 * pc;
+        if (col >= n_out) return;  // N is a multiple of 16: the pair is inside or outside together
+        const float o0 = v0 * p_gamma, o1 = v1 * p_gamma;
+        if (a.y_dtype == TAMD_F32) {
+          ((float *)a.y)[p_dst + col] = o0;
+          ((float *)a.y)[p_dst + col + 1] = o1;
+        } else {
+          uint16_t *yp = (uint16_t *)a.y + p_dst + col;
+          if (((uintptr_t)yp & 3) == 0) *(uint32_t *)yp = to_16(o0) | (to_16(o1) << 16);
+          else yp[0] = (uint16_t)to_16(o0), yp[1] = (uint16_t)to_16(o1);
+        }
+      }
+    };
+    int slot = 0;
+#pragma unroll 1
+    for (int s = 0; s < total_stages; ++s) {
+      __syncthreads();  // the partial sums of stage s - 1 and the bias of stage s are visible
+#if !(TAMD_ABL & 1)
+      if (s > 0) finish((s - 1) & 1);
+#endif
+      if (c_blk < blk0 || c_cg == n_cg) {
+        if (c_cg == n_cg) c_cg = 0;
+        load_rows(++c_blk);
+      }
+      // this unit's bias and row data travel to the next iteration
+      const uint2 braw = *(const uint2 *)(lds + slot * S::STAGE + S::CODE_BYTES + S::SC_BYTES + pc * 8);
+      p_bias0 = to_f32(braw.x), p_bias1 = to_f32(braw.y);
+      p_beta = row_beta, p_gamma = row_gamma, p_dst = row_dst;
+      p_col0 = c_cg * 16;
+      ++c_cg;
+      slot = slot + 1 == S::RING ? 0 : slot + 1;
     }
-    const uint32_t sb = lds_base + slot * S::STAGE;
-    const v4i_t dw = live ? rw : rw0;
+    __syncthreads();
+    finish((total_stages - 1) & 1);
+  } else if (wave8 >= 4) {
+    // =========================================================================== copying waves
+    // Wave 4 requests the first half of a unit's code image and its scale image, wave 5 the second half
+    // and the bias.  A wave that issues copies stalls whenever the memory pipeline is full, which is
+    // exactly how these two keep it full; nothing else runs on them.
+    const int half = wave8 - 4;
+    const v4i_t rw = make_rsrc(a.w, kOob), rs = make_rsrc(a.w_mx_scale, kOob), rb = make_rsrc(a.bias, kOob);
+    // empty descriptors (no records: every lane out of range) for copies past the end of the range,
+    // issued so that the count of outstanding copies per stage never changes
+    const v4i_t rw0 = make_rsrc(a.w, 0), rs0 = make_rsrc(a.w_mx_scale, 0), rb0 = make_rsrc(a.bias, 0);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const int bias_esz = a.bias_dtype == TAMD_F32 ? 4 : 2;
+    constexpr int NP = 2 * SS;  // code pieces (1 KB) per copying wave
+    // per-lane source offsets never change: a unit's codes, scales and bias are linear images
+    uint32_t w_voff[NP];
 #pragma unroll
-    for (int i = 0; i < SS; ++i) {
-      const uint32_t m0v = sb + (wave * SS + i / 4 * 4) * 1024;
-      const uint32_t so = i_wbase + (uint32_t)(i / 4) * 4096u;
-      if (i % 4 == 0) dma16_at<0, true>(dw, m0v, w_voff[i], so);
-      if (i % 4 == 1) dma16_at<1024, false>(dw, m0v, w_voff[i], so);
-      if (i % 4 == 2) dma16_at<2048, false>(dw, m0v, w_voff[i], so);
-      if (i % 4 == 3) dma16_at<3072, false>(dw, m0v, w_voff[i], so);
+    for (int i = 0; i < NP; ++i) {
+      const uint32_t lin = (uint32_t)(half * NP + i) * 1024u + lane * 16u;
+      w_voff[i] = lin < 16u * col_bytes ? (uint32_t)(half * NP) * 1024u + lane * 16u : kOob;  // piece i adds i*1024 itself
     }
-    if (wave < 2) {
-      dma16(live ? rs : rs0, sb + S::CODE_BYTES + wave * 1024, x_voff, i_sbase);
+    uint32_t x_voff[2];
+    if (half == 0) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) x_voff[q] = q * 1024u + lane * 16u < (uint32_t)(16 * G) ? q * 1024u + lane * 16u : kOob;
     } else {
-      const uint32_t dst = sb + S::CODE_BYTES + S::SC_BYTES + (wave - 2) * 256;  // an empty copy writes zeros
-      if (bias_esz == 4) dma4(live ? rb : rb0, dst, x_voff, i_bbase);
-      else dma2(live ? rb : rb0, dst, x_voff, i_bbase);
+      x_voff[0] = (a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
+      x_voff[1] = kOob;
     }
-    ++i_cg, --i_left;
-    i_wbase += 16u * col_bytes, i_sbase += (uint32_t)(16 * G), i_bbase += (uint32_t)(16 * bias_esz);
-  };
-
-  // ---- compute side state: the row block whose activations sit in registers
-  frag_t areg[SS * 4];
-  int c_blk = blk0 - 1, c_cg = cg0;
-  Block cb;
-  float row_beta = 1.f, row_gamma = 1.f;
-  int64_t row_dst = -1;
-  const int kb = 4 * SS * wave;  // first e8m0 group of this wave's K slice
-  auto load_block = [&](int blk) {
-    get_block(blk, cb);
-    int rc = c16 < cb.rows ? c16 : cb.rows - 1;
-    rc = cb.row0 + (rc < 0 ? 0 : rc);
-    const int64_t src = a.gather_indx ? (int64_t)a.gather_indx[rc] : (int64_t)rc;
-    const uint16_t *xr = (const uint16_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+    int i_blk = blk0 - 1, i_cg = cg0, i_left = total_stages;
+    uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0;
+    auto issue = [&](int slot) {
+      const bool live = i_left > 0;
+      if (live && (i_blk < blk0 || i_cg == n_cg)) {
+        if (i_cg == n_cg) i_cg = 0;
+        ++i_blk;
+        Block b;
+        get_block(i_blk, b);
+        const int e = __builtin_amdgcn_readfirstlane(b.expert);  // keeps the running offsets in scalar registers
+        i_wbase = (uint32_t)((int64_t)e * a.w_stride_e) + (uint32_t)i_cg * 16u * col_bytes;
+        i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e) + (uint32_t)(i_cg * 16 * G);
+        i_bbase = (uint32_t)(((int64_t)e * a.bias_stride_e + i_cg * 16) * bias_esz);
+      }
+      const uint32_t sb = lds_base + slot * S::STAGE;
+      const v4i_t dw = live ? rw : rw0;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const uint32_t m0v = sb + (half * NP + i / 4 * 4) * 1024;
+        const uint32_t so = i_wbase + (uint32_t)(i / 4) * 4096u;
+        if (i % 4 == 0) dma16_at<0, true>(dw, m0v, w_voff[i], so);
+        if (i % 4 == 1) dma16_at<1024, false>(dw, m0v, w_voff[i], so);
+        if (i % 4 == 2) dma16_at<2048, false>(dw, m0v, w_voff[i], so);
+        if (i % 4 == 3) dma16_at<3072, false>(dw, m0v, w_voff[i], so);
+      }
+      if (half == 0) {
+        dma16(live ? rs : rs0, sb + S::CODE_BYTES, x_voff[0], i_sbase);
+        dma16(live ? rs : rs0, sb + S::CODE_BYTES + 1024, x_voff[1], i_sbase);
+      } else {
+        const uint32_t dst = sb + S::CODE_BYTES + S::SC_BYTES;
+        if (bias_esz == 4) dma4(live ? rb : rb0, dst, x_voff[0], i_bbase);
+        else dma2(live ? rb : rb0, dst, x_voff[0], i_bbase);
+      }
+      ++i_cg, --i_left;
+      i_wbase += 16u * col_bytes, i_sbase += (uint32_t)(16 * G), i_bbase += (uint32_t)(16 * bias_esz);
+    };
+    // stage s lives in slot s % RING and is requested RING - 1 stages ahead
+    int i_slot = 0;
+#pragma unroll 1
+    for (int s = 0; s < S::RING - 1; ++s) {
+      issue(i_slot);
+      i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
+    }
+#pragma unroll 1
+    for (int s = 0; s < total_stages; ++s) {
+      // copies complete in order: once at most RING - 2 stages' worth are outstanding, stage s has landed
+      if (half == 0) wait_vmcnt<(S::RING - 2) * (NP + 2)>();
+      else wait_vmcnt<(S::RING - 2) * (NP + 1)>();
+      __syncthreads();  // publishes stage s; every wave is done with stage s - 1, whose slot is refilled now
+      issue(i_slot);
+      i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
+    }
+    __syncthreads();
+    wait_vmcnt<0>();  // the empty copies issued past the end still write (zeros) to LDS
+  } else {
+    // =========================================================================== compute waves
+    const int c16 = lane % 16, g = lane / 16;
+    const int kb = 4 * SS * wave;  // first e8m0 group of this wave's K slice
+    frag_t areg[SS * 4];           // this wave's K slice of the block's rows, row c16
+    int c_blk = blk0 - 1, c_cg = cg0;
+    auto load_block = [&](int blk) {
+      Block cb;
+      get_block(blk, cb);
+      int rc = c16 < cb.rows ? c16 : cb.rows - 1;
+      rc = cb.row0 + (rc < 0 ? 0 : rc);
+      const int64_t src = a.gather_indx ? (int64_t)a.gather_indx[rc] : (int64_t)rc;
+      const uint16_t *xr = (const uint16_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+#pragma unroll
+      for (int j = 0; j < SS; ++j) {
+        const int kg = kb + 4 * j + g;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          uint4 v = make_uint4(0, 0, 0, 0);
+          if (kg < G && cb.rows > 0) v = *(const uint4 *)(xr + 32 * kg + 8 * u);
+          areg[j * 4 + u] = __builtin_bit_cast(frag_t, v);
+        }
+      }
+    };
+    // per-lane LDS offsets of this wave's K slice inside a stage (beyond K: group 0 with scale 1.0 --
+    // the activations there are zero, the weight operand only has to stay finite)
+    uint32_t b_loff[SS], s_loff[SS];
+    bool kvalid[SS];
 #pragma unroll
     for (int j = 0; j < SS; ++j) {
       const int kg = kb + 4 * j + g;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (kg < G && cb.rows > 0) v = *(const uint4 *)(xr + 32 * kg + 8 * u);
-        areg[j * 4 + u] = __builtin_bit_cast(frag_t, v);
+      kvalid[j] = kg < G;
+      b_loff[j] = (uint32_t)c16 * col_bytes + (kvalid[j] ? kg : 0) * 16;
+      s_loff[j] = (uint32_t)(S::CODE_BYTES + c16 * G + (kvalid[j] ? kg : 0));
+    }
+    int slot = 0;
+#pragma unroll 1
+    for (int s = 0; s < total_stages; ++s) {
+      __syncthreads();
+      if (c_blk < blk0 || c_cg == n_cg) {
+        if (c_cg == n_cg) c_cg = 0;
+        load_block(++c_blk);
       }
-    }
-    const bool rv = er < cb.rows;
-    const int erow = cb.row0 + (rv ? er : 0);
-    row_beta = (a.betas && rv) ? a.betas[erow] : 1.0f;
-    row_gamma = (a.gammas && rv) ? a.gammas[erow] : 1.0f;
-    row_dst = rv ? (a.scatter_indx ? (int64_t)a.scatter_indx[erow] : (int64_t)erow) : -1;
-    row_dst = row_dst < 0 ? -1 : (int64_t)cb.z * a.y_stride_z + row_dst * a.y_stride_m;
-  };
-  // per-lane LDS offsets of this wave's K slice inside a stage (beyond K: group 0 with scale 1.0 --
-  // the activations there are zero, the weight operand only has to stay finite)
-  uint32_t b_loff[SS], s_loff[SS];
-  bool kvalid[SS];
+      ++c_cg;
+      const uint8_t *img = lds + slot * S::STAGE;
+      uint4 raw[SS];
+      uint32_t sby[SS];
 #pragma unroll
-  for (int j = 0; j < SS; ++j) {
-    const int kg = kb + 4 * j + g;
-    kvalid[j] = kg < G;
-    b_loff[j] = (uint32_t)c16 * col_bytes + (kvalid[j] ? kg : 0) * 16;
-    s_loff[j] = (uint32_t)(S::CODE_BYTES + c16 * G + (kvalid[j] ? kg : 0));
-  }
-
-  float flex = 1.0f;
-  if (a.x_scale) flex *= *a.x_scale;
-  if (a.w_scale) flex *= *a.w_scale;
-  const bool has_limit = a.act_has_limit != 0;
-  const int n_out = SW ? N / 2 : N;
-  const int red_idx = ((er >> 2) * 16 + ec) * 4 + (er & 3);
-
-  // what the deferred epilogue of the previous unit needs
-  float p_bias = 0.f, p_beta = 1.f, p_gamma = 1.f;
-  int64_t p_dst = -1;
-  int p_col0 = 0;
-  auto epilogue = [&](int buf) {
-    const float *rbuf = red + buf * 1024 + red_idx;
-    const float sum = (rbuf[0] + rbuf[256]) + (rbuf[512] + rbuf[768]);
-    float v = (sum * flex + p_bias * p_beta) * a.out_alpha;
-    int col = p_col0 + ec;
-    bool store = p_dst >= 0;
-    if constexpr (SW) {
-      const float other = __shfl_xor(v, 1);
-      v = swiglu_fast(v, other, a.act_alpha, a.act_limit, has_limit);
-      store = store && (ec & 1) == 0;
-      col >>= 1;
-    }
-    v *= p_gamma;
-    if (store && col < n_out) {
-      const int64_t at = p_dst + col;
-      if (a.y_dtype == TAMD_F32) ((float *)a.y)[at] = v;
-      else ((uint16_t *)a.y)[at] = (uint16_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
-    }
-  };
-
-  // ---- the ring: stage s lives in slot s % RING and is requested RING - 1 stages ahead
-  int i_slot = 0;
-#pragma unroll 1
-  for (int s = 0; s < S::RING - 1; ++s) {
-    issue(i_slot);
-    i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
-  }
-  int slot = 0;
-#pragma unroll 1
-  for (int s = 0; s < total_stages; ++s) {
-    // copies complete in order: once at most RING - 2 stages' worth are outstanding, stage s has landed
-    wait_vmcnt<(S::RING - 2) * S::DMA_PER_STAGE>();
-    __syncthreads();  // stage s and the partial sums of stage s - 1 are visible; slot (s - 1) % RING is free
-    issue(i_slot);
-    i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
-    if (s > 0) epilogue((s - 1) & 1);
-    if (c_blk < blk0 || c_cg == n_cg) {
-      if (c_cg == n_cg) c_cg = 0;
-      load_block(++c_blk);
-    }
-
-    const uint8_t *img = lds + slot * S::STAGE;
-    f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+      for (int j = 0; j < SS; ++j) {
+        raw[j] = *(const uint4 *)(img + b_loff[j]);
+        sby[j] = img[s_loff[j]];
+      }
+      // four independent accumulation chains keep dependent MFMAs apart
+      f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
 #pragma unroll
-    for (int j = 0; j < SS; ++j) {
-      const uint4 r = *(const uint4 *)(img + b_loff[j]);
-      const uint32_t sbyte = kvalid[j] ? (uint32_t)img[s_loff[j]] : 127u;
-      const float sc = bits_to_f32(sbyte << 23);
-      acc0 = Mma16<XDT>::mma(areg[j * 4 + 0], M::expand(r.x, sc), acc0);
-      acc1 = Mma16<XDT>::mma(areg[j * 4 + 1], M::expand(r.y, sc), acc1);
-      acc0 = Mma16<XDT>::mma(areg[j * 4 + 2], M::expand(r.z, sc), acc0);
-      acc1 = Mma16<XDT>::mma(areg[j * 4 + 3], M::expand(r.w, sc), acc1);
+      for (int j = 0; j < ((TAMD_ABL & 2) ? 1 : SS); ++j) {
+        const float sc = bits_to_f32((kvalid[j] ? sby[j] : 127u) << 23);
+        acc0 = Mma16<XDT>::mma(areg[j * 4 + 0], M::expand(raw[j].x, sc), acc0);
+        acc1 = Mma16<XDT>::mma(areg[j * 4 + 1], M::expand(raw[j].y, sc), acc1);
+        acc2 = Mma16<XDT>::mma(areg[j * 4 + 2], M::expand(raw[j].z, sc), acc2);
+        acc3 = Mma16<XDT>::mma(areg[j * 4 + 3], M::expand(raw[j].w, sc), acc3);
+      }
+      *(f32x4_t *)(red + (s & 1) * 1024 + wave * 256 + lane * 4) = (acc0 + acc1) + (acc2 + acc3);
+      slot = slot + 1 == S::RING ? 0 : slot + 1;
     }
-    *(f32x4_t *)(red + (s & 1) * 1024 + wave * 256 + lane * 4) = acc0 + acc1;
-
-    // carry this unit's epilogue operands to the next iteration
-    const uint32_t braw = *(const uint32_t *)(img + S::CODE_BYTES + S::SC_BYTES + ec * 4);
-    p_bias = a.bias == nullptr ? 0.f
-                               : (a.bias_dtype == TAMD_F32 ? bits_to_f32(braw)
-                                                           : (a.bias_dtype == TAMD_BF16 ? bits_to_f32(braw << 16)
-                                                                                        : f16_bits_to_f32((uint16_t)braw)));
-    p_beta = row_beta, p_gamma = row_gamma, p_dst = row_dst;
-    p_col0 = c_cg * 16;
-    ++c_cg;
-    slot = slot + 1 == S::RING ? 0 : slot + 1;
+    __syncthreads();
   }
-  __syncthreads();
-  epilogue((total_stages - 1) & 1);
-  wait_vmcnt<0>();  // the empty copies issued past the end still write (zeros) to LDS
 }
 
 // Whether the streaming kernel covers the problem: K contiguous and dense per column for codes and
@@ -356,8 +418,7 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
 
 template <int XDT, int ACT, int SS>
 int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int WGS_PER_CU = TAMD_STREAM_WGS_PER_CU;
-  constexpr int RING_FIT = ((WGS_PER_CU == 1 ? 156 : 80) * 1024 - 8192) / (4 * SS * 1024 + 2048 + 512);
+  constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + 2048 + 256);
   constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
   const int n_cg = (a.N + 15) / 16;
   const int64_t upper = (int64_t)grid_m * n_cg;
@@ -366,11 +427,11 @@ int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   hipError_t e = hipGetDevice(&dev);
   if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (e != hipSuccess) return (int)e;
-  const int wgs = (int)(upper < cus * WGS_PER_CU ? upper : cus * WGS_PER_CU);
-  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, WGS_PER_CU>;
+  const int wgs = (int)(upper < cus ? upper : cus);
+  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING>;
   e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   if (e != hipSuccess) return (int)e;
-  kern<<<dim3((unsigned)wgs), 256, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
+  kern<<<dim3((unsigned)wgs), 512, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
   return launch_status();
 }
 
