@@ -279,7 +279,7 @@ struct MetaPlan {
   int CH;
   int nbits;
   int64_t n_chunks, n_blocks;
-  int64_t off_chunk_pref, off_block_tot, off_col_offs, off_n_valid, total;
+  int64_t off_chunk_pref, off_block_tot, off_block_off, off_col_offs, off_n_valid, total;
 };
 
 inline MetaPlan make_meta_plan(int64_t n_indx, int E) {
@@ -295,7 +295,8 @@ inline MetaPlan make_meta_plan(int64_t n_indx, int E) {
   if (p.n_blocks < 1) p.n_blocks = 1;
   p.off_chunk_pref = 0;
   p.off_block_tot = p.n_blocks * ch * (int64_t)E;
-  p.off_col_offs = p.off_block_tot + p.n_blocks * (int64_t)E;
+  p.off_block_off = p.off_block_tot + p.n_blocks * (int64_t)E;
+  p.off_col_offs = p.off_block_off + p.n_blocks * (int64_t)E;
   p.off_n_valid = p.off_col_offs + E;
   p.total = p.off_n_valid + 1;
   return p;
@@ -320,52 +321,228 @@ inline int launch_bitmatrix_metadata(const void *indx, int is16, int64_t n, int 
 // ---------------------------------------------------------------------------
 // ragged tensor metadata
 // ---------------------------------------------------------------------------
-// One block.  Wave r < 6 scans row r of the offsets table (r = 0: slice offsets,
-// r >= 1: block offsets for block size 8 << r); then all 16 waves fill the
-// schedule, one (block size, slice) pair at a time with lanes over its blocks.
+// Row r of the offsets table: r = 0 slice offsets, r >= 1 block offsets for block size 8 << r.
+// Wave r < 6 of a workgroup scans row r (64 slices per step with a running carry) into `tab`
+// (pitch S + 1) and, when `offs` is given, into global memory.
+TAMD_DEVICE void ragged_scan_rows(const int32_t *sizes, int S, int32_t *tab, int32_t *offs, int64_t offs_pitch) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (wave >= 6) return;
+  const int sh = wave == 0 ? 0 : wave + 3;
+  int32_t *trow = tab + (int64_t)wave * (S + 1);
+  int32_t *grow = offs ? offs + (int64_t)wave * offs_pitch : nullptr;
+  int carry = 0;
+  for (int s0 = 0; s0 < S; s0 += kWave) {
+    const int s = s0 + lane;
+    const int v = s < S ? ((sizes[s] + ((1 << sh) - 1)) >> sh) : 0;
+    int inc = v;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int t = __shfl_up(inc, o);
+      if (lane >= o) inc += t;
+    }
+    if (s < S) {
+      trow[s] = carry + inc - v;
+      if (grow) grow[s] = carry + inc - v;
+    }
+    carry += __shfl(inc, kWave - 1);
+  }
+  if (lane == 0) {
+    trow[S] = carry;
+    if (grow) grow[S] = carry;
+  }
+}
+
+// Schedule entry j of block size index b is ((j - block_offs[s]) << 16) | s for the slice s whose block
+// range holds j (binary search in the scanned row; empty slices are skipped by the search), -1 past
+// the last block.  Entries [first, first + count) of the flattened [5][max_blocks] table.
+TAMD_DEVICE void ragged_fill_schedule(const int32_t *tab, int S, int32_t *sched, int64_t sched_pitch, int max_blocks,
+                                      int64_t first, int64_t count) {
+  for (int64_t idx = first + threadIdx.x; idx < first + count; idx += blockDim.x) {
+    const int b = (int)(idx / max_blocks), j = (int)(idx - (int64_t)b * max_blocks);
+    const int32_t *row = tab + (int64_t)(b + 1) * (S + 1);
+    int val = -1;
+    if (j < row[S]) {
+      int lo = 0, hi = S - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (row[mid + 1] <= j) lo = mid + 1;
+        else hi = mid;
+      }
+      val = ((j - row[lo]) << 16) + lo;
+    }
+    sched[(int64_t)b * sched_pitch + j] = val;
+  }
+}
+
+// Every workgroup scans the (small) size vector into its own LDS copy of the table, workgroup 0 also
+// writes it out, and the schedule entries are split evenly over the workgroups.
 __global__ __launch_bounds__(1024) void ragged_kernel(const int32_t *__restrict__ sizes, int S,
                                                       int32_t *__restrict__ offs, int64_t offs_pitch,
                                                       int32_t *__restrict__ sched, int64_t sched_pitch, int max_blocks) {
-  __shared__ int totals[6];
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  if (wave < 6) {
-    const int sh = wave == 0 ? 0 : wave + 3;
-    int32_t *row = offs + (int64_t)wave * offs_pitch;
-    int carry = 0;
-    for (int s0 = 0; s0 < S; s0 += kWave) {
-      int s = s0 + lane;
-      int v = s < S ? ((sizes[s] + ((1 << sh) - 1)) >> sh) : 0;
-      int inc = v;
-#pragma unroll
-      for (int o = 1; o < kWave; o <<= 1) {
-        int t = __shfl_up(inc, o);
-        if (lane >= o) inc += t;
-      }
-      if (s < S) row[s] = carry + inc - v;
-      carry += __shfl(inc, kWave - 1);
-    }
-    if (lane == 0) {
-      row[S] = carry;
-      totals[wave] = carry;
-    }
-  }
-  __threadfence_block();
+  extern __shared__ int32_t tab[];  // [6][S + 1]
+  ragged_scan_rows(sizes, S, tab, blockIdx.x == 0 ? offs : nullptr, offs_pitch);
   __syncthreads();
-  for (int p = wave; p < 5 * S; p += 16) {
-    const int b = p / S, s = p - b * S;
-    const int sh = b + 4;
-    const int nb = (sizes[s] + ((1 << sh) - 1)) >> sh;
-    const int start = offs[(int64_t)(b + 1) * offs_pitch + s];
-    int32_t *row = sched + (int64_t)b * sched_pitch;
-    for (int i = lane; i < nb; i += kWave) {
-      int j = start + i;
-      if (j < max_blocks) row[j] = (i << 16) + s;
+  const int64_t total = 5 * (int64_t)max_blocks;
+  const int64_t per = (total + gridDim.x - 1) / gridDim.x;
+  const int64_t first = per * blockIdx.x;
+  if (first < total) ragged_fill_schedule(tab, S, sched, sched_pitch, max_blocks, first, per < total - first ? per : total - first);
+}
+
+// Second of three launches for larger index arrays: the prefix sums over the per-workgroup histograms
+// (as scan_kernel) merged with the ragged tables.  Every workgroup repeats the small scans into its own
+// LDS and fills its share of the schedule; workgroup 0 alone writes the scan results.  The prefix over
+// workgroups goes to `block_off` (not in place: the other workgroups still read `block_tot`).
+__global__ __launch_bounds__(1024) void scan_ragged_kernel(int E, int n_blocks, const int32_t *__restrict__ block_tot,
+                                                           int32_t *__restrict__ block_off, int32_t *__restrict__ col_sum,
+                                                           int32_t *__restrict__ col_offs, int32_t *__restrict__ n_valid,
+                                                           int32_t *__restrict__ offs, int64_t offs_pitch,
+                                                           int32_t *__restrict__ sched, int64_t sched_pitch, int max_blocks) {
+  extern __shared__ int32_t sm[];
+  int32_t *csum = sm;             // [E]
+  int32_t *tab = csum + E;        // [6][E + 1]
+  int32_t *scr = tab + 6 * (E + 1);
+  const bool lead = blockIdx.x == 0;
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 1024) {
+    const int e = e0 + threadIdx.x;
+    int run = 0;
+    if (e < E) {
+#pragma unroll 4
+      for (int b = 0; b < n_blocks; ++b) {
+        const int t = block_tot[(int64_t)b * E + e];
+        if (lead) block_off[(int64_t)b * E + e] = run;
+        run += t;
+      }
+      csum[e] = run;
+      if (lead) col_sum[e] = run;
+    }
+    int total;
+    const int ex = block_excl_scan_1024(run, total, scr);
+    if (lead && e < E) col_offs[e] = carry + ex;
+    carry += total;
+    __syncthreads();
+  }
+  if (lead && threadIdx.x == 0) *n_valid = carry;
+  ragged_scan_rows(csum, E, tab, lead ? offs : nullptr, offs_pitch);
+  __syncthreads();
+  const int64_t total_e = 5 * (int64_t)max_blocks;
+  const int64_t per = (total_e + gridDim.x - 1) / gridDim.x;
+  const int64_t first = per * blockIdx.x;
+  if (first < total_e)
+    ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, first, per < total_e - first ? per : total_e - first);
+}
+
+// ---------------------------------------------------------------------------
+// all routing metadata in one workgroup
+// ---------------------------------------------------------------------------
+// For index arrays small enough that the per-chunk histogram fits LDS (n/64 * E ints): histogram,
+// the three prefix sums, the ordering and the ragged tables without leaving the workgroup --
+// one launch instead of four, which is what the cost of routing is made of at these sizes.
+__global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict__ indx, int is16, int n, int E, int k,
+                                                          int nbits, int NC, int P, int32_t *__restrict__ col_sum,
+                                                          int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
+                                                          int32_t *__restrict__ gather, int32_t *__restrict__ offs,
+                                                          int64_t offs_pitch, int32_t *__restrict__ sched,
+                                                          int64_t sched_pitch, int max_blocks) {
+  extern __shared__ int32_t sm[];
+  int32_t *hist = sm;                         // [NC][E]  counts, then exclusive prefix over chunks
+  int32_t *csum = hist + (int64_t)NC * E;     // [E]
+  int32_t *coff = csum + E;                   // [E]
+  int32_t *psum = coff + E;                   // [P][E]   partial sums of chunk ranges
+  int32_t *tab = psum + (int64_t)P * E;       // [6][E + 1]
+  int32_t *scr = tab + 6 * (E + 1);           // [17]
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  for (int i = tid; i < NC * E; i += 1024) hist[i] = 0;
+  __syncthreads();
+  // 1. per-chunk histogram.  A wave takes its chunks eight at a time so that eight index loads are in
+  // flight together (one workgroup has nothing else to hide their latency with).
+  for (int c0 = wave; c0 < NC; c0 += 16 * 8) {
+    int ev[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = (c0 + 16 * u) * 64 + lane;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? load_indx(indx, is16, i) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + 16 * u;
+      if (c >= NC) break;
+      const int e = ev[u];
+      const bool valid = e >= 0 && e < E;
+      const uint64_t same = same_id_mask(e, valid, nbits);
+      if (valid && (same & lanemask_lt()) == 0) hist[c * E + e] = __popcll(same);
     }
   }
-  for (int b = 0; b < 5; ++b) {
-    int32_t *row = sched + (int64_t)b * sched_pitch;
-    for (int j = totals[b + 1] + (int)threadIdx.x; j < max_blocks; j += 1024) row[j] = -1;
+  __syncthreads();
+  // 2. exclusive prefix over chunks for every expert: P chunk ranges per expert, two passes
+  const int per = (NC + P - 1) / P;
+  for (int t = tid; t < P * E; t += 1024) {
+    const int part = t / E, e = t - part * E;
+    int run = 0;
+    for (int c = part * per; c < NC && c < (part + 1) * per; ++c) run += hist[c * E + e];
+    psum[part * E + e] = run;
   }
+  __syncthreads();
+  for (int t = tid; t < P * E; t += 1024) {
+    const int part = t / E, e = t - part * E;
+    int run = 0;
+    for (int q = 0; q < part; ++q) run += psum[q * E + e];
+    for (int c = part * per; c < NC && c < (part + 1) * per; ++c) {
+      const int v = hist[c * E + e];
+      hist[c * E + e] = run;
+      run += v;
+    }
+    if (part == P - 1) {
+      csum[e] = run;
+      col_sum[e] = run;
+    }
+  }
+  __syncthreads();
+  // 3. exclusive prefix over experts
+  int carry = 0;
+  for (int e0 = 0; e0 < E; e0 += 1024) {
+    const int e = e0 + tid;
+    int total;
+    const int ex = block_excl_scan_1024(e < E ? csum[e] : 0, total, scr);
+    if (e < E) coff[e] = carry + ex;
+    carry += total;
+    __syncthreads();
+  }
+  const int nv = carry;
+  // 4. placement
+  for (int c0 = wave; c0 < NC; c0 += 16 * 8) {
+    int ev[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = (c0 + 16 * u) * 64 + lane;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? load_indx(indx, is16, i) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + 16 * u;
+      if (c >= NC) break;
+      const int i = c * 64 + lane;
+      const int e = ev[u];
+      const bool valid = e >= 0 && e < E;
+      const uint64_t same = same_id_mask(e, valid, nbits);
+      if (valid) {
+        const int pos = coff[e] + hist[c * E + e] + __popcll(same & lanemask_lt());
+        row_sorted[i] = pos;
+        col_sorted[pos] = i;
+        if (gather) gather[pos] = i / k;
+      } else if (i < n) {
+        row_sorted[i] = -1;
+      }
+      if (i >= nv && i < n) {
+        col_sorted[i] = -1;
+        if (gather) gather[i] = 0;  // trunc(-1 / k)
+      }
+    }
+  }
+  // 5. ragged tables of the histogram
+  ragged_scan_rows(csum, E, tab, offs, offs_pitch);
+  __syncthreads();
+  ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, 0, 5 * (int64_t)max_blocks);
 }
 
 }  // namespace tamd
@@ -411,7 +588,14 @@ extern "C" int tamd_bitmatrix_metadata(const void *indx, int indx_is_int16, int6
 
 static int ragged_launch(const int32_t *slice_sizes, int n_slices, int32_t *offs, int64_t offs_pitch,
                          int32_t *schedule, int64_t sched_pitch, int max_n_blocks, hipStream_t st) {
-  ragged_kernel<<<1, 1024, 0, st>>>(slice_sizes, n_slices, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
+  const size_t lds = 6 * (size_t)(n_slices + 1) * 4;
+  if (lds > 150 * 1024) return TAMD_E_UNSUPPORTED;  // more than ~6000 slices
+  hipError_t e = hipFuncSetAttribute((const void *)ragged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  int64_t wgs = (5 * (int64_t)max_n_blocks + 4095) / 4096;  // about four entries per thread
+  wgs = wgs < 1 ? 1 : (wgs > 256 ? 256 : wgs);
+  ragged_kernel<<<dim3((unsigned)wgs), 1024, lds, st>>>(slice_sizes, n_slices, offs, offs_pitch, schedule, sched_pitch,
+                                                      max_n_blocks);
   return launch_status();
 }
 
@@ -451,6 +635,42 @@ extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_
   if (max_n_blocks < 0 || offs_pitch < n_cols + 1 || sched_pitch < max_n_blocks) return TAMD_E_INVALID;
   if (!col_sum || !workspace || !offs || (max_n_blocks > 0 && !schedule)) return TAMD_E_INVALID;
   if (n_indx > 0 && (!indx || !col_sorted_indx || !row_sorted_indx)) return TAMD_E_INVALID;
+  {
+    // one workgroup does it all when the per-chunk histogram fits its LDS
+    const int64_t NC = (n_indx + 63) / 64 > 0 ? (n_indx + 63) / 64 : 1;
+    int64_t P = 1024 / n_cols;
+    P = P < 1 ? 1 : (P > NC ? NC : P);
+    const int64_t ints = NC * n_cols + 2 * (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1) + 17;
+    if (NC <= 64 && ints * 4 <= 156 * 1024) {  // beyond ~4096 entries one CU is slower than three launches
+      int nbits = 0;
+      while ((1 << nbits) < n_cols) ++nbits;
+      hipError_t e = hipFuncSetAttribute((const void *)meta_fused_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return (int)e;
+      meta_fused_kernel<<<1, 1024, (size_t)ints * 4, (hipStream_t)stream>>>(
+          indx, indx_is_int16, (int)n_indx, n_cols, k, nbits, (int)NC, (int)P, col_sum, col_sorted_indx, row_sorted_indx,
+          gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
+      return launch_status();
+    }
+  }
+  const size_t sr_lds = ((size_t)n_cols + 6 * ((size_t)n_cols + 1) + 17) * 4;
+  if (sr_lds <= 150 * 1024) {
+    // three launches: histograms per workgroup, scans + ragged tables, placement
+    hipStream_t st = (hipStream_t)stream;
+    MetaPlan p = make_meta_plan(n_indx, n_cols);
+    hist_kernel<<<dim3((unsigned)p.n_blocks), 256, (size_t)p.CH * n_cols * 4, st>>>(
+        indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, workspace + p.off_chunk_pref, workspace + p.off_block_tot);
+    hipError_t e = hipFuncSetAttribute((const void *)scan_ragged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    int64_t wgs = (5 * (int64_t)max_n_blocks + 4095) / 4096;
+    wgs = wgs < 1 ? 1 : (wgs > 64 ? 64 : wgs);
+    scan_ragged_kernel<<<dim3((unsigned)wgs), 1024, sr_lds, st>>>(
+        n_cols, (int)p.n_blocks, workspace + p.off_block_tot, workspace + p.off_block_off, col_sum,
+        workspace + p.off_col_offs, workspace + p.off_n_valid, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
+    order_kernel<<<dim3((unsigned)p.n_blocks), 256, 0, st>>>(
+        indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, k, workspace + p.off_chunk_pref, workspace + p.off_block_off,
+        workspace + p.off_col_offs, workspace + p.off_n_valid, col_sorted_indx, row_sorted_indx, gather_indx);
+    return launch_status();
+  }
   RaggedCtx ctx{col_sum, n_cols, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, (hipStream_t)stream};
   return launch_bitmatrix_metadata(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx,
                                    row_sorted_indx, gather_indx, workspace, (hipStream_t)stream, ragged_between, &ctx);
