@@ -208,11 +208,20 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   // ---- scales of the whole tile, once: 256 columns x G bytes, contiguous in memory
   const int tile_cols = N - t.n0 < BLOCK_N ? N - t.n0 : BLOCK_N;
   if constexpr (SC_LDS) {
-    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(s_base + (int64_t)t.n0 * G), 0, (uint32_t)(tile_cols * G), 0x00020000);
-    const int n_dw = (BLOCK_N * G + 3) / 4;
-    for (int i = tid; i < n_dw; i += 256)
-      ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
+    const uint8_t *sc_src = s_base + (int64_t)t.n0 * G;
+    if ((((uintptr_t)sc_src) & 15) == 0 && (N * G) % 16 == 0) {
+      // by DMA, 1 KB per instruction: in flight together with the first activation / weight stages and
+      // awaited with them at the first barrier of the K loop
+      const v4i_t rs = make_rsrc(sc_src, (uint32_t)((N - t.n0) * G));
+      const uint32_t lds_sc_addr = lds_base + 2 * A_STAGE + B_BYTES;
+      for (int i = wave; i * 1024 < BLOCK_N * G; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
+    } else {
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
+                                                                        0x00020000);
+      const int n_dw = (BLOCK_N * G + 3) / 4;
+      for (int i = tid; i < n_dw; i += 256)
+        ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
+    }
   }
 
   // ---- activation DMA: one instruction per 32-row fragment, lane -> (row 8w + lane/8, slot lane%8)
@@ -506,7 +515,7 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
   // scales of a tile are staged in LDS when they are dense ([N][K/32]) and two workgroups still fit a CU
   const int64_t G = a.K / 32;
-  const int64_t sc_bytes = (BLOCK_N * G + 15) / 16 * 16;
+  const int64_t sc_bytes = (BLOCK_N * G + 1023) / 1024 * 1024;  // whole 1 KB copies
   const bool dense_sc = a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
                         aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0;
   const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;

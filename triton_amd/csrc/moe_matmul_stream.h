@@ -23,9 +23,6 @@
 #pragma once
 #include "moe_matmul_impl.h"
 
-#ifndef TAMD_ABL
-#define TAMD_ABL 0  // timing experiments only: 1 = no epilogue, 2 = one super step, 4 = no wait for the copies
-#endif
 
 namespace tamd {
 
@@ -230,9 +227,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
 #pragma unroll 1
     for (int s = 0; s < total_stages; ++s) {
       __syncthreads();  // the partial sums of stage s - 1 and the bias of stage s are visible
-#if !(TAMD_ABL & 1)
       if (s > 0) finish((s - 1) & 1);
-#endif
       if (c_blk < blk0 || c_cg == n_cg) {
         if (c_cg == n_cg) c_cg = 0;
         load_rows(++c_blk);
@@ -384,7 +379,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       // four independent accumulation chains keep dependent MFMAs apart
       f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
 #pragma unroll
-      for (int j = 0; j < ((TAMD_ABL & 2) ? 1 : SS); ++j) {
+      for (int j = 0; j < SS; ++j) {
         const float sc = bits_to_f32((kvalid[j] ? sby[j] : 127u) << 23);
         acc0 = Mma16<XDT>::mma(areg[j * 4 + 0], M::expand(raw[j].x, sc), acc0);
         acc1 = Mma16<XDT>::mma(areg[j * 4 + 1], M::expand(raw[j].y, sc), acc1);
