@@ -16,12 +16,9 @@ TAMD_DEVICE uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, 
 
 TAMD_DEVICE float bf16_bits_to_f32(uint32_t h) { return bits_to_f32(h << 16); }
 
-// float32 -> bfloat16 bits, round to nearest even, NaN kept quiet.
+// float32 -> bfloat16 bits, round to nearest even, NaN kept quiet (one v_cvt_pk_bf16_f32 on gfx950).
 TAMD_DEVICE uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = f32_to_bits(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return u >> 16;
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 
 TAMD_DEVICE float f16_bits_to_f32(uint32_t h) {
