@@ -110,14 +110,29 @@ struct Tile {
 };
 
 template <int BLOCK_M, int EXTRA>
-TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid_total, Tile &t) {
+TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid_total, int group_m, Tile &t) {
   // XCD-aware remap: hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
   // contiguous range of tiles so neighbours (same expert, adjacent columns) share one L2.
   const int64_t per_xcd = (grid_total + 7) / 8;
   int64_t pid = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (pid >= grid_total) return false;
-  int pid_m = (int)(pid / grid_n);
-  int pid_n = (int)(pid - (int64_t)pid_m * grid_n);
+  // Tiles are walked in groups of `group_m` row blocks: row block fastest inside a group, then the
+  // column tile.  With many row blocks per expert the workgroups running together then share one
+  // column tile of weights while the group's activation rows stay in L2; group_m = 1 is the plain
+  // row-block-major order (right when an expert has only a block or two).
+  int pid_m, pid_n;
+  if (group_m > 1) {
+    const int grid_m = (int)(grid_total / grid_n);
+    const int64_t in_group = (int64_t)group_m * grid_n;
+    const int first_m = (int)(pid / in_group) * group_m;
+    const int size_m = grid_m - first_m < group_m ? grid_m - first_m : group_m;
+    const int r = (int)(pid - (pid / in_group) * in_group);
+    pid_m = first_m + r % size_m;
+    pid_n = r / size_m;
+  } else {
+    pid_m = (int)(pid / grid_n);
+    pid_n = (int)(pid - (int64_t)pid_m * grid_n);
+  }
   t.n0 = pid_n * BLOCK_N;
   t.z = 0;
   int slice_rows;
@@ -478,10 +493,10 @@ struct TileShape {
 
 // BM: block size of the ragged schedule the kernel consumes (16..128).
 template <int XDT, int BM, int ACT, bool SC_LDS>
-TAMD_DEVICE void tile_entry(const tamd_matmul_args &a, int grid_n, int64_t grid_total, uint8_t *lds) {
+TAMD_DEVICE void tile_entry(const tamd_matmul_args &a, int grid_n, int64_t grid_total, int group_m, uint8_t *lds) {
   typedef TileShape<XDT, BM> S;
   Tile t;
-  if (!locate_tile<BM, S::EXTRA>(a, grid_n, grid_total, t)) return;
+  if (!locate_tile<BM, S::EXTRA>(a, grid_n, grid_total, group_m, t)) return;
   const int nfr = (t.rows + 31) / 32;  // active row fragments (workgroup uniform)
 #define TAMD_CASE(n)                                                                 \
   case n:                                                                            \
@@ -492,15 +507,17 @@ TAMD_DEVICE void tile_entry(const tamd_matmul_args &a, int grid_n, int64_t grid_
 }
 
 template <int XDT, int BM, int ACT, bool SC_LDS>
-__global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+__global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total,
+                                                                  int group_m) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  tile_entry<XDT, BM, ACT, SC_LDS>(a, grid_n, grid_total, lds);
+  tile_entry<XDT, BM, ACT, SC_LDS>(a, grid_n, grid_total, group_m, lds);
 }
 
 template <int XDT, int BM, int ACT, bool SC_LDS>
-__global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+__global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total,
+                                                                 int group_m) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  tile_entry<XDT, BM, ACT, SC_LDS>(a, grid_n, grid_total, lds);
+  tile_entry<XDT, BM, ACT, SC_LDS>(a, grid_n, grid_total, group_m, lds);
 }
 
 template <int XDT, int BM, int ACT>
@@ -521,7 +538,7 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;
   size_t lds_bytes = PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
   if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;
-  void (*kern)(tamd_matmul_args, int, int64_t);
+  void (*kern)(tamd_matmul_args, int, int64_t, int);
   if constexpr (is_fp8(XDT))
     kern = sc_in_lds ? mm_x8_mxfp4_kernel<XDT, BM, ACT, true> : mm_x8_mxfp4_kernel<XDT, BM, ACT, false>;
   else
@@ -529,7 +546,14 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   // raising the dynamic LDS limit is idempotent, so doing it on every launch keeps the entry point stateless
   hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   if (e != hipSuccess) return (int)e;
-  kern<<<dim3((unsigned)launch), 256, lds_bytes, st>>>(a, grid_n, total);
+  // row blocks walked together: as many as one expert (or batch entry) has, while their activation
+  // rows (BM x K each) fit comfortably in one XCD's 4 MB L2
+  const int64_t rows_per_slice = a.block_schedule ? a.M / a.n_experts : a.M;
+  int64_t group_m = rows_per_slice / BM;
+  const int64_t fit = (int64_t)(2.5 * 1024 * 1024) / ((int64_t)BM * a.K * (is_fp8(XDT) ? 1 : 2));
+  group_m = group_m > fit ? fit : group_m;
+  group_m = group_m < 1 ? 1 : (group_m > 16 ? 16 : group_m);
+  kern<<<dim3((unsigned)launch), 256, lds_bytes, st>>>(a, grid_n, total, (int)group_m);
   return launch_status();
 }
 
