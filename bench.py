@@ -25,7 +25,7 @@ PEAK_MXFP4_TFLOPS = 10100.0
 
 # HBM bytes per launch of the dominant kernel (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00 KiB from rocprofv3 --pmc,
 # factors from the hbm_copy workload).  Counters cannot be read from inside this process; re-measure after kernel changes.
-MEASURED_TRAFFIC = {"fc1_prefill": 1536778240, "fc1_decode": 1558978560}
+MEASURED_TRAFFIC = {"fc1_prefill": 1574256640, "fc1_decode": 976203776, "fc2_combine": 1473740800}
 
 WORKLOADS = {
     # name: (T, E, k, K, N, swiglu)
@@ -296,7 +296,8 @@ def main():
     else:
         roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
                     frac=round(tflops_kernel / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
-    roof["kernel"] = "mm_x16_mxfp4_kernel"
+    # row blocks of 16 (few rows per expert) run the weight-streaming kernel, everything else the tiled one
+    roof["kernel"] = "mm_stream16_kernel" if rows <= 16 * E else "mm_x16_mxfp4_kernel"
     roof["kernel_ms"] = round(kernel_ms, 4)
     roof["algorithmic_bytes"] = abytes
     roof["algorithmic_flops"] = flops
