@@ -84,6 +84,12 @@ def matmul_ref(a, b, bias, slice_sizes=None, gather_indx=None, scatter_indx=None
     return y
 
 
+def actual_scale_ref(y: torch.Tensor, out_dtype) -> torch.Tensor:
+    """max|y| / max_finite(out_dtype): what a flexpoint output records as its actual scale
+    (compute_actual_scale, matmul.py:812-821 of the reference)."""
+    return (y.float().abs().max() / torch.finfo(out_dtype).max).reshape(1)
+
+
 def swiglu_ref(a: torch.Tensor, alpha: float, limit):
     """Interleaved SwiGLU, swiglu.py:89-100: gate = even columns clamped from
     above, linear = odd columns clamped to [-limit, limit];

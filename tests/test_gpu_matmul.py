@@ -311,3 +311,107 @@ def test_decode_shape_of_the_baseline(device):
     ref = MR.matmul_ref(x, rv, bias, slice_sizes=rr["col_sum"], gather_indx=rr["gather_indx"], b_mx_scale=rs,
                         fused_swiglu=(1.702, 7.0))
     check(out, ref)
+
+
+# ---------------------------------------------------------------------------- flexpoint (fp8) output
+
+
+def test_fp8_output_conversion_is_exact(device):
+    """One-hot activations times a per-row gate weight give single float32 products deq(W)[k, n] * gamma[r]: the
+    fp8 output must equal torch's own float32 -> float8_e4m3fn cast of them bit for bit (round to nearest even,
+    subnormals, NaN beyond the range without saturation, the largest finite value with it)."""
+    from triton_amd.matmul import OutFlexData
+    torch.manual_seed(0)
+    K, N, M = 64, 256, 64
+    w = torch.randn(K, N) * 4
+    v, s, rv, rs = quantize_w(w, device)
+    from oracle.mxfp_ref import upcast_from_mxfp_ref
+    deq = upcast_from_mxfp_ref(rv, rs, torch.float32, axis=0)
+    x = torch.eye(K, dtype=torch.bfloat16)[:M]
+    gammas = torch.exp(torch.linspace(-12, 6, M)).float()
+    for saturate in (False, True):
+        actual = torch.zeros(1, device=device)
+        flex = FlexCtx(out_data=OutFlexData(torch.float8_e4m3fn, torch.ones(1, device=device), actual, None))
+        pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, flex_ctx=flex,
+                             flexpoint_saturate_inf=saturate)
+        out = matmul(x.to(device), v, None, precision_config=pc, gammas=gammas.to(device))
+        assert out.dtype == torch.float8_e4m3fn
+        prod = deq[:M] * gammas[:, None]
+        want = (prod.clamp(-448, 448) if saturate else prod).to(torch.float8_e4m3fn)
+        # a -0.0 weight summed with the +0.0 products of the other K positions is +0.0: ignore the sign of zero
+        pos_zero = lambda t: torch.where(t == 0x80, torch.zeros_like(t), t)
+        assert torch.equal(pos_zero(out.cpu().view(torch.uint8)), pos_zero(want.view(torch.uint8)))
+        assert actual.item() == pytest.approx(float(prod.abs().max()) / 448.0, rel=1e-6)
+
+
+@pytest.mark.parametrize("block_m", [16, 128])
+@pytest.mark.parametrize("act", [False, True])
+def test_fp8_output_with_expected_scale(block_m, act, device):
+    """FC1-style problem emitting fp8 with a flexpoint scale: values = result / expected_scale cast to e4m3, and
+    the actual scale is max|result| / 448 (reference: float_to_flex / compute_actual_scale)."""
+    from triton_amd.matmul import OutFlexData
+    torch.manual_seed(1)
+    E, K, N = 5, 320, 384
+    sizes = torch.tensor([3, 0, 16, 140, 9], dtype=torch.int32)
+    M = int(sizes.sum())
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    expected = torch.tensor([0.03125], device=device)
+    actual = torch.zeros(1, device=device)
+    flex = FlexCtx(out_data=OutFlexData(torch.float8_e4m3fn, expected, actual, None))
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, flex_ctx=flex,
+                         flexpoint_saturate_inf=True)
+    with scoped_opt_flags_constraints({"block_m": block_m}):
+        out = matmul(x.to(device), v, bias.to(device), md, precision_config=pc,
+                     fused_activation=swiglu_act(1.702, 7.0) if act else None)
+    ref32 = MR.matmul_ref(x.float(), rv, bias, slice_sizes=sizes, b_mx_scale=rs, fused_swiglu=(1.702, 7.0) if act else None)
+    want = (ref32 / 0.03125).clamp(-448, 448)
+    got = out.float().cpu()
+    # fp8 has 3 mantissa bits: one step of the result grid is 2^-3 relative; allow one step plus the GEMM tolerance
+    assert ((got - want).abs() <= 0.13 * want.abs() + 0.02 / 0.03125).all()
+    assert_close(want.to(torch.float8_e4m3fn).float(), got, maxtol=7e-2, rmstol=2e-2, verbose=False)
+    assert actual.item() == pytest.approx(MR.actual_scale_ref(ref32, torch.float8_e4m3fn).item(), rel=2e-3)
+
+
+def test_moe_mlp_chain_with_fp8_intermediate(device):
+    """routing -> FC1 (gather, bias, SwiGLU) emitting fp8 with a flexpoint scale -> FC2 consuming those fp8 rows
+    with the same scale (gate weights, scatter) -> top-k combine; against the oracle chained the same way."""
+    from triton_amd.matmul import OutFlexData
+    from triton_amd.reduce import reduce
+    torch.manual_seed(0)
+    T, E, k, H, I = 192, 8, 2, 256, 512
+    logits = torch.randn(T, E)
+    x = torch.randn(T, H).to(torch.bfloat16)
+    w1 = torch.randn(E, H, 2 * I) * 0.05
+    w2 = torch.randn(E, I, H) * 0.05
+    b1, b2 = torch.randn(E, 2 * I) * 0.1, torch.randn(E, H) * 0.1
+    v1, s1, rv1, rs1 = quantize_w(w1, device)
+    v2, s2, rv2, rs2 = quantize_w(w2, device)
+    r = routing(logits.to(device), k)
+    rr = RR.routing_ref(logits, k)
+    mid_scale = torch.tensor([1.0 / 64], device=device)
+    actual = torch.zeros(1, device=device)
+    pc1 = PrecisionConfig(b_mx_scale=s1, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, flexpoint_saturate_inf=True,
+                          flex_ctx=FlexCtx(out_data=OutFlexData(torch.float8_e4m3fn, mid_scale, actual, None)))
+    h = matmul(x.to(device), v1, b1.to(device), r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1,
+               fused_activation=swiglu_act(1.702, 7.0))
+    assert h.dtype == torch.float8_e4m3fn and tuple(h.shape) == (T * k, I)
+    pc2 = PrecisionConfig(b_mx_scale=s2, b_microblock_size=32, out_dtype=torch.bfloat16,
+                          flex_ctx=FlexCtx(lhs_data=InFlexData(torch.float8_e4m3fn, mid_scale)))
+    gam = r.expert_sorted_gate_weights
+    y = matmul(h, v2, b2.to(device), r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2, gammas=gam)
+    z, _ = reduce(y.view(T, k, H), dim=1)
+    # oracle: same chain, the fp8 rounding of the intermediate included (taken from the kernel's own fp8 rows, which
+    # are checked against the float32 oracle first)
+    h_ref32 = MR.matmul_ref(x.float(), rv1, b1, slice_sizes=rr["col_sum"], gather_indx=rr["gather_indx"], b_mx_scale=rs1,
+                            fused_swiglu=(1.702, 7.0))
+    want_h = (h_ref32 * 64).clamp(-448, 448)
+    assert ((h.float().cpu() - want_h).abs() <= 0.13 * want_h.abs() + 0.64).all()
+    assert actual.item() == pytest.approx(MR.actual_scale_ref(h_ref32, torch.float8_e4m3fn).item(), rel=2e-3)
+    y_ref = MR.matmul_ref(h.cpu(), rv2, b2, slice_sizes=rr["col_sum"], scatter_indx=rr["scatter_indx"], b_mx_scale=rs2,
+                          a_flex_scale=mid_scale.cpu(), gammas=gam.cpu()).to(torch.bfloat16)
+    check(y, y_ref)
+    assert torch.equal(z.cpu(), MR.reduce_ref(y.cpu().view(T, k, H), 1))

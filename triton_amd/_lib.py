@@ -49,6 +49,7 @@ class MatmulArgs(C.Structure):
         ("x_stride_z", C.c_int64), ("y_stride_z", C.c_int64),
         ("activation", C.c_int), ("act_alpha", C.c_float), ("act_limit", C.c_float), ("act_has_limit", C.c_int),
         ("force_variant", C.c_int), ("x_rows", C.c_int64),
+        ("y_expected_scale", C.c_void_p), ("y_actual_scale", C.c_void_p), ("y_saturate_inf", C.c_int),
     ]
 
 

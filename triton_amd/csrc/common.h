@@ -28,6 +28,25 @@ TAMD_DEVICE uint32_t f32_to_f16_bits(float f) {
   return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
+// float32 -> OCP e4m3fn byte, round to nearest even.  Magnitudes that round beyond 448 (>= 464) give the
+// largest finite code when `saturate`, NaN otherwise (what a plain cast does); NaN stays NaN.
+TAMD_DEVICE uint32_t f32_to_e4m3_bits(float f, bool saturate) {
+  const uint32_t u = f32_to_bits(f), sign = (u >> 24) & 0x80u, mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) return sign | 0x7Fu;
+  if (mag >= 0x43E80000u) return sign | (saturate ? 0x7Eu : 0x7Fu);  // 464.0f
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xFFu;
+}
+
+// Largest finite value of an output type, and the running |x| maximum kept as float bits so that NaN
+// (above +inf as an integer) survives the maximum (flexpoint.py:119-146 of the reference).
+TAMD_DEVICE float max_finite_of(int dt) {
+  return dt == TAMD_FP8_E4M3 ? 448.0f : (dt == TAMD_F16 ? 65504.0f : (dt == TAMD_BF16 ? 3.3895313892515355e38f : 3.4028234663852886e38f));
+}
+TAMD_DEVICE uint32_t absmax_bits(uint32_t run, float v) {
+  const uint32_t b = f32_to_bits(v) & 0x7FFFFFFFu;
+  return b > run ? b : run;
+}
+
 // OCP e4m3fn byte -> float32 (exact).
 TAMD_DEVICE float e4m3_bits_to_f32(uint32_t b) {
   uint32_t s = (b & 0x80u) << 24;

@@ -418,8 +418,18 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
   const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
   const bool has_limit = a.act_has_limit != 0;
-  const bool staged = a.y_dtype != TAMD_F32;
-  uint16_t *ob = (uint16_t *)lds;  // [rows][OUT_COLS]
+  const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
+  const bool staged = osz < 4;
+  // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
+  const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
+  const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
+  const float out_max = max_finite_of(a.y_dtype);
+  uint32_t amax = 0;
+  auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
+    return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v)
+                                  : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
+  };
+  uint8_t *ob = lds;  // [rows][OUT_COLS] outputs of osz bytes
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < NFR; ++i) {
@@ -439,14 +449,24 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
         for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
       }
+      if (a.y_actual_scale && r < t.rows) {
+#pragma unroll
+        for (int p = 0; p < NO; ++p)
+          if (out_col0 + p < n_out) amax = absmax_bits(amax, o[p]);
+      }
+#pragma unroll
+      for (int p = 0; p < NO; ++p) {
+        o[p] *= inv_expected;
+        if (clamp_out) o[p] = __builtin_fminf(__builtin_fmaxf(o[p], -out_max), out_max);
+      }
       if (staged) {
-        uint16_t *dstl = ob + r * OUT_COLS + wave * 32 * NO + c32 * NO;
-        if constexpr (NO == 2) {
-          uint32_t w2 = a.y_dtype == TAMD_BF16 ? (f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[NO - 1]) << 16))
-                                               : (f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[NO - 1]) << 16));
-          *(uint32_t *)dstl = w2;
+        uint8_t *dstl = ob + (r * OUT_COLS + wave * 32 * NO + c32 * NO) * osz;
+        if (osz == 2) {
+          if constexpr (NO == 2) *(uint32_t *)dstl = narrow(o[0]) | (narrow(o[NO - 1]) << 16);
+          else *(uint16_t *)dstl = (uint16_t)narrow(o[0]);
         } else {
-          *dstl = (uint16_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(o[0]) : f32_to_f16_bits(o[0]));
+          if constexpr (NO == 2) *(uint16_t *)dstl = (uint16_t)(narrow(o[0]) | (narrow(o[NO - 1]) << 8));
+          else *dstl = (uint8_t)narrow(o[0]);
         }
       } else if (r < t.rows) {
         int64_t dst = t.start_m + t.off_m + r;
@@ -460,23 +480,38 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       }
     }
   }
+  if (a.y_actual_scale) {
+    // wave maximum, then one atomic per wave; positive floats order like their bit patterns
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
+      amax = other > amax ? other : amax;
+    }
+    if (lane == 0) {
+      amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
+      const float sc = __builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f);
+      atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(sc));
+    }
+  }
   if (staged) {
     __syncthreads();
-    constexpr int CPR = OUT_COLS / 8;  // 16-byte chunks per tile row
-    const int n_chunks = t.rows * CPR;
+    const int epc = 16 / osz;                 // outputs per 16-byte chunk
+    const int cpr = OUT_COLS / epc;           // chunks per tile row
+    const int n_chunks = t.rows * cpr;
     for (int id = tid; id < n_chunks; id += 256) {
-      const int r = id / CPR, c = (id - r * CPR) * 8;
+      const int r = id / cpr, c = (id - r * cpr) * epc;
       int64_t dst = t.start_m + t.off_m + r;
       if (a.scatter_indx) dst = a.scatter_indx[dst];
       if (dst < 0) continue;
       const int gcol = tile_out0 + c;
       if (gcol >= n_out) continue;
-      uint16_t *yp = (uint16_t *)a.y + (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol;
-      const uint16_t *sp = ob + r * OUT_COLS + c;
-      if (gcol + 8 <= n_out && ((uintptr_t)yp & 15) == 0) {
+      uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * osz;
+      const uint8_t *sp = ob + (r * OUT_COLS + c) * osz;
+      if (gcol + epc <= n_out && ((uintptr_t)yp & 15) == 0) {
         *(uint4 *)yp = *(const uint4 *)sp;
       } else {
-        for (int e = 0; e < 8 && gcol + e < n_out; ++e) yp[e] = sp[e];
+        const int n_b = (n_out - gcol < epc ? n_out - gcol : epc) * osz;
+        for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
       }
     }
   }

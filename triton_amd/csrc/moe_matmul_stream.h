@@ -193,8 +193,20 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
                                                            : (a.bias_dtype == TAMD_BF16 ? bits_to_f32(raw << 16)
                                                                                         : f16_bits_to_f32((uint16_t)raw)));
     };
-    auto to_16 = [&](float v) {
-      return (uint32_t)(a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v)) & 0xFFFFu;
+    const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);
+    auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
+      return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) & 0xFFFFu
+                                    : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) & 0xFFFFu : f32_to_e4m3_bits(v, false));
+    };
+    // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
+    const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
+    const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
+    const float out_max = max_finite_of(a.y_dtype);
+    uint32_t amax = 0;
+    auto flex_out = [&](float v) {
+      if (a.y_actual_scale) amax = absmax_bits(amax, v);
+      v *= inv_expected;
+      return clamp_out ? __builtin_fminf(__builtin_fmaxf(v, -out_max), out_max) : v;
     };
     auto finish = [&](int buf) {
       const float *rbuf = red + buf * 1024 + red_idx;
@@ -206,20 +218,25 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       if constexpr (SW) {
         const int col = (p_col0 >> 1) + pc;
         if (col >= n_out) return;
-        const float o = swiglu_fast(v0, v1, a.act_alpha, a.act_limit, has_limit) * p_gamma;
-        if (a.y_dtype == TAMD_F32) ((float *)a.y)[p_dst + col] = o;
-        else ((uint16_t *)a.y)[p_dst + col] = (uint16_t)to_16(o);
+        const float o = flex_out(swiglu_fast(v0, v1, a.act_alpha, a.act_limit, has_limit) * p_gamma);
+        if (osz == 4) ((float *)a.y)[p_dst + col] = o;
+        else if (osz == 2) ((uint16_t *)a.y)[p_dst + col] = (uint16_t)narrow(o);
+        else ((uint8_t *)a.y)[p_dst + col] = (uint8_t)narrow(o);
       } else {
         const int col = p_col0 + 2 * pc;
         if (col >= n_out) return;  // N is a multiple of 16: the pair is inside or outside together
-        const float o0 = v0 * p_gamma, o1 = v1 * p_gamma;
-        if (a.y_dtype == TAMD_F32) {
+        const float o0 = flex_out(v0 * p_gamma), o1 = flex_out(v1 * p_gamma);
+        if (osz == 4) {
           ((float *)a.y)[p_dst + col] = o0;
           ((float *)a.y)[p_dst + col + 1] = o1;
-        } else {
+        } else if (osz == 2) {
           uint16_t *yp = (uint16_t *)a.y + p_dst + col;
-          if (((uintptr_t)yp & 3) == 0) *(uint32_t *)yp = to_16(o0) | (to_16(o1) << 16);
-          else yp[0] = (uint16_t)to_16(o0), yp[1] = (uint16_t)to_16(o1);
+          if (((uintptr_t)yp & 3) == 0) *(uint32_t *)yp = narrow(o0) | (narrow(o1) << 16);
+          else yp[0] = (uint16_t)narrow(o0), yp[1] = (uint16_t)narrow(o1);
+        } else {
+          uint8_t *yp = (uint8_t *)a.y + p_dst + col;
+          if (((uintptr_t)yp & 1) == 0) *(uint16_t *)yp = (uint16_t)(narrow(o0) | (narrow(o1) << 8));
+          else yp[0] = (uint8_t)narrow(o0), yp[1] = (uint8_t)narrow(o1);
         }
       }
     };
@@ -242,6 +259,18 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
     }
     __syncthreads();
     finish((total_stages - 1) & 1);
+    if (a.y_actual_scale) {
+      // wave maximum, then one atomic per wave; positive floats order like their bit patterns
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
+        amax = other > amax ? other : amax;
+      }
+      if (lane == 0) {
+        amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
+        atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(__builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f)));
+      }
+    }
   } else if (wave8 >= 4) {
     // =========================================================================== copying waves
     // Wave 4 requests the first half of a unit's code image and its scale image, wave 5 the second half

@@ -111,9 +111,13 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if precision_config.a_mx_scale is not None:
         raise NotImplementedError("microscaled activations are not built")
     flex = precision_config.flex_ctx
-    if flex.out_data.expected_scale is not None or flex.out_data.actual_scale is not None \
-            or flex.acc_data.scale is not None:
-        raise NotImplementedError("flexpoint output scaling is not built")
+    if flex.acc_data.scale is not None:
+        raise NotImplementedError("accumulator flex scale is not built")
+    if flex.out_data.checksum_scale is not None:
+        raise NotImplementedError("flexpoint checksum is not built")
+    for sc in (flex.out_data.expected_scale, flex.out_data.actual_scale):
+        if sc is not None and (sc.numel() != 1 or sc.dtype != torch.float32):
+            raise NotImplementedError("per-batch flexpoint output scales are not built (one float32 value expected)")
     # ---- weights
     b_scale = precision_config.b_mx_scale
     if not isinstance(b, Tensor):
@@ -145,9 +149,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
     out_dtype = precision_config.out_dtype or a.dtype
-    if out_dtype.itemsize == 1:
-        raise NotImplementedError("fp8 outputs need flexpoint output scaling, which is not built: "
-                                  "set precision_config.out_dtype to bfloat16 / float16 / float32")
+    if out_dtype.itemsize == 1 and out_dtype != torch.float8_e4m3fn:
+        raise NotImplementedError(f"{out_dtype} outputs are not built (float8_e4m3fn is)")
     rows_out = M
     if gather_indx is not None:
         rows_out = gather_indx.shape[0]
@@ -227,6 +230,11 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     args.y_stride_m, args.y_stride_z = out.stride(1), out.stride(0)
     args.M, args.N, args.K, args.n_experts = M, N, K, n_slices
     args.x_rows = a.shape[-2]
+    if flex.out_data.expected_scale is not None:
+        args.y_expected_scale = flex.out_data.expected_scale.data_ptr()
+    if flex.out_data.actual_scale is not None:
+        args.y_actual_scale = flex.out_data.actual_scale.data_ptr()
+    args.y_saturate_inf = int(precision_config.flexpoint_saturate_inf)
     args.gather_indx, args.scatter_indx = i32(gather_indx), i32(scatter_indx)
     if ragged:
         md = a_ragged_metadata
