@@ -415,3 +415,49 @@ def test_moe_mlp_chain_with_fp8_intermediate(device):
                           a_flex_scale=mid_scale.cpu(), gammas=gam.cpu()).to(torch.bfloat16)
     check(y, y_ref)
     assert torch.equal(z.cpu(), MR.reduce_ref(y.cpu().view(T, k, H), 1))
+
+
+# ---------------------------------------------------------------------------- unquantised 16-bit weights
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 2880, 128), (16, 64, 64), (33, 96, 200), (130, 192, 520), (1, 8, 8), (300, 2048, 1024)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("k_contiguous", [False, True])
+def test_dense_16bit_weights(M, K, N, dtype, k_contiguous, device):
+    """(256, 2880, 128) is the gate matmul of the MoE block (hidden -> expert logits)."""
+    torch.manual_seed(0)
+    x = torch.randn(M, K).to(dtype)
+    w = (torch.randn(K, N) * 0.05).to(dtype)
+    bias = torch.randn(N)
+    wd = w.to(device)
+    if k_contiguous:
+        wd = wd.T.contiguous().T  # same values, unit stride along K
+        assert wd.stride() == (1, K)
+    out = matmul(x.to(device), wd, bias.to(device))
+    ref = MR.matmul_ref(x, w, bias)
+    assert out.dtype == dtype and tuple(out.shape) == (M, N)
+    check(out, ref)
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 64])
+@pytest.mark.parametrize("act", [False, True])
+def test_ragged_16bit_weights(block_m, act, device):
+    torch.manual_seed(1)
+    E, K, N, M = 6, 320, 392, 500
+    sizes = torch.tensor([0, 5, 130, 16, 249, 100], dtype=torch.int32)
+    x = torch.randn(M + 3, K).to(torch.bfloat16)
+    w = (torch.randn(E, K, N) * 0.05).to(torch.bfloat16)
+    bias = torch.randn(E, N)
+    gather = torch.randint(0, M + 3, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::11] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    out_init = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=device)
+    with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+        out = matmul(x.to(device), w.to(device), bias.to(device), md, gather_indx=gather.to(device),
+                     scatter_indx=scatter.to(device), gammas=gammas.to(device),
+                     fused_activation=swiglu_act(1.702, 7.0) if act else None, c=out_init)
+    ref = MR.matmul_ref(x, w, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, gammas=gammas,
+                        fused_swiglu=(1.702, 7.0) if act else None)
+    check(out, ref)

@@ -34,7 +34,7 @@ def build(force=True, verbose=False):
     os.makedirs(objdir, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in srcs]
-    deps = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "moe_matmul_impl.h"), os.path.join(CSRC, "moe_matmul_stream.h"),
+    deps = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "moe_matmul_impl.h"), os.path.join(CSRC, "moe_matmul_stream.h"), os.path.join(CSRC, "moe_matmul_dense.h"),
             os.path.join(HERE, "..", "include", "triton_amd.h")]
     todo = []
     for s, o in zip(srcs, objs):

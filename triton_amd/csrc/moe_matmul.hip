@@ -7,6 +7,8 @@ namespace tamd {
 int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int dispatch_mm_w16_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int dispatch_mm_w16_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 }  // namespace tamd
 
 using namespace tamd;
@@ -53,6 +55,19 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     if (a.x_dtype == TAMD_BF16) return dispatch_mm_bf16(a, block_m, grid_m, st);
     if (a.x_dtype == TAMD_F16) return dispatch_mm_f16(a, block_m, grid_m, st);
     return dispatch_mm_fp8e4m3(a, block_m, grid_m, st);
+  }
+  if ((a.x_dtype == TAMD_BF16 || a.x_dtype == TAMD_F16) && a.w_dtype == a.x_dtype) {
+    // unquantised weights of the activations' type
+    int block_m, grid_m;
+    if (ragged) {
+      block_m = a.block_m;
+      grid_m = a.grid_m;
+    } else {
+      block_m = a.force_variant ? a.force_variant : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128);
+      grid_m = ((a.M + block_m - 1) / block_m) * a.n_experts;
+    }
+    if (a.x_dtype == TAMD_BF16) return dispatch_mm_w16_bf16(a, block_m, grid_m, st);
+    return dispatch_mm_w16_f16(a, block_m, grid_m, st);
   }
   return TAMD_E_UNSUPPORTED;
 }

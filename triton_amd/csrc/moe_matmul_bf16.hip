@@ -1,5 +1,7 @@
 // Instantiates the grouped matmul kernels for one activation type: the streaming kernel for row blocks of
-// 16 (moe_matmul_stream.h) and the tiled kernel for everything else (moe_matmul_impl.h).
+// 16 (moe_matmul_stream.h), the tiled MXFP4 kernel for everything else (moe_matmul_impl.h), and the kernel for
+// unquantised weights of the same type (moe_matmul_dense.h).
+#include "moe_matmul_dense.h"
 #include "moe_matmul_stream.h"
 
 namespace tamd {
@@ -9,5 +11,9 @@ int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStre
     return launch_stream16<TAMD_BF16, TAMD_ACT_NONE>(a, grid_m, st);
   }
   return dispatch_x16<TAMD_BF16>(a, block_m, grid_m, st);
+}
+
+int dispatch_mm_w16_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  return dispatch_w16<TAMD_BF16>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

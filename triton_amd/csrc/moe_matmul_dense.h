@@ -1,0 +1,209 @@
+// Grouped / dense matmul with unquantised 16-bit weights (bf16 x bf16, f16 x f16): the gate matmul and
+// every caller of `matmul` that passes plain weights.  Same tile decomposition, activation staging and
+// epilogue as the MXFP4 kernel of moe_matmul_impl.h; only the weight path differs:
+//
+//   * K-contiguous weights (w_stride_k == 1, the layout of the quantised weights): a stage holds
+//     [256 columns][64 K] = 128 bytes per column, copied by DMA exactly like activation rows and read
+//     as 16-byte MFMA fragments;
+//   * N-contiguous weights (w_stride_n == 1, the usual row-major [K, N]): a stage holds
+//     [64 K][256 columns] as it lies in memory (512 bytes per K row); a lane gathers the 8 K values of
+//     its column with 2-byte LDS reads.  The MFMA wants K-contiguous operands on both sides, so one of
+//     the two has to be transposed somewhere; doing it on the LDS read costs no extra pass.
+//
+// One workgroup per CU (the two 32 KB weight stages need the LDS); not a tuned kernel -- the unquantised
+// products on this path are small next to the expert matmuls.
+#pragma once
+#include "moe_matmul_impl.h"
+
+namespace tamd {
+
+constexpr int W16_STAGE = 256 * 128;  // bytes of one weight stage in either layout
+
+template <int XDT, int NFR, int LDS_ROWS, int ACT, bool WKC>
+TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t *lds) {
+  typedef Mma<XDT> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int KA = 64;
+  constexpr int A_STAGE = LDS_ROWS * A_ROW_BYTES;
+  constexpr uint32_t kOob = 0x7FFFFFFFu;
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave, lane = tid % kWave;
+  const int c32 = lane % 32, h = lane / 32;
+  const int K = a.K, N = a.N;
+
+  const v4i_t rx = make_rsrc((const uint8_t *)a.x + (int64_t)t.z * a.x_stride_z * 2, kOob);
+  // the descriptor ends with the expert's weights: a copy that starts inside and runs past the end
+  // (partial last chunk of columns) delivers zeros for the part outside
+  const int64_t w_span = (WKC ? (int64_t)N * a.w_stride_n : (int64_t)K * a.w_stride_k) * 2;
+  const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e * 2, (uint32_t)w_span);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const uint32_t lds_b = lds_base + 2 * A_STAGE;
+
+  // ---- activation DMA (as in run_tile): lane -> (row 8w + lane/8, slot lane%8)
+  const int a_rin = wave * 8 + lane / 8;
+  const int a_chunk = (lane % 8) ^ ((a_rin >> 1) & 7);
+  uint32_t a_off[NFR];
+#pragma unroll
+  for (int i = 0; i < NFR; ++i) {
+    const int r = i * 32 + a_rin;
+    const int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
+    const uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
+    a_off[i] = src * (uint32_t)(a.x_stride_m * 2) + a_chunk * 16;
+  }
+  // ---- weight DMA: 8 instructions per wave and stage
+  uint32_t w_off[8];
+  int w_chunk[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if constexpr (WKC) {
+      // LDS row p = wave*64 + j*8 + lane/8 holds tile column wave*64 + 2*(q%32) + q/32 (q = p%64) so that a lane's
+      // two fragments are a gate / linear pair; 16-byte chunks swizzled like activation rows
+      const int q = j * 8 + lane / 8;
+      const int col = t.n0 + wave * 64 + 2 * (q % 32) + q / 32;
+      w_chunk[j] = (lane % 8) ^ (((wave * 64 + q) >> 1) & 7);
+      w_off[j] = col < N ? (uint32_t)col * (uint32_t)(a.w_stride_n * 2) + w_chunk[j] * 16 : kOob;
+    } else {
+      // K rows 16w + 2j, 16w + 2j + 1 of the stage, 32 chunks of 8 columns each
+      const int col = t.n0 + 8 * (lane % 32);
+      w_chunk[j] = wave * 16 + 2 * j + lane / 32;  // K row inside the stage
+      // N is a multiple of 8 here; the lane's half (lane/32) of the K row pair goes into the vector offset, the
+      // pair's first row into the wave-uniform scalar offset
+      w_off[j] = col + 8 <= N ? (uint32_t)col * 2u + (uint32_t)(lane / 32) * (uint32_t)(a.w_stride_k * 2) : kOob;
+    }
+  }
+
+  f32x16_t acc[NFR][NF];
+#pragma unroll
+  for (int i = 0; i < NFR; ++i)
+#pragma unroll
+    for (int f = 0; f < NF; ++f)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[i][f][j] = 0.f;
+
+  const int n_k = (K + KA - 1) / KA;
+  auto issue = [&](int it) {  // clamped: past the end the last stage is copied again (never read)
+    it = it < n_k ? it : n_k - 1;
+    const int kb = it * KA;
+    const uint32_t akill = kb + a_chunk * 8 < K ? 0u : kOob;
+    const uint32_t sa = lds_base + (it & 1) * A_STAGE + wave * 8 * A_ROW_BYTES;
+#pragma unroll
+    for (int i = 0; i < NFR; ++i) dma16(rx, sa + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * 2);
+    const uint32_t sb = lds_b + (it & 1) * W16_STAGE;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (WKC) {
+        const uint32_t kill = kb + w_chunk[j] * 8 < K ? 0u : kOob;
+        dma16(rw, sb + (wave * 64 + j * 8) * 128, w_off[j] | kill, kb * 2);
+      } else {
+        const int k = kb + w_chunk[j];
+        const uint32_t kill = k < K ? 0u : kOob;
+        dma16(rw, sb + (wave * 16 + 2 * j) * 512, w_off[j] | kill,
+              (uint32_t)((int64_t)(kb + wave * 16 + 2 * j) * a.w_stride_k * 2));
+      }
+    }
+  };
+
+  auto compute = [&](int it) {
+    const uint8_t *abuf = lds + (it & 1) * A_STAGE;
+    const uint8_t *bbuf = lds + 2 * A_STAGE + (it & 1) * W16_STAGE;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      frag_t af[NFR];
+      const int aslot = (h * 4 + s) ^ ((c32 >> 1) & 7);
+#pragma unroll
+      for (int i = 0; i < NFR; ++i) af[i] = *(const frag_t *)(abuf + (i * 32 + c32) * A_ROW_BYTES + aslot * 16);
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        frag_t bf;
+        if constexpr (WKC) {
+          const int p = wave * 64 + f * 32 + c32;
+          bf = *(const frag_t *)(bbuf + p * 128 + (((h * 4 + s) ^ ((p >> 1) & 7)) * 16));
+        } else {
+          const uint16_t *colp = (const uint16_t *)bbuf + (wave * 64 + c32 * NF + f);
+          uint32_t w[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int k = (h * 4 + s) * 8 + 2 * e;
+            w[e] = (uint32_t)colp[k * 256] | ((uint32_t)colp[(k + 1) * 256] << 16);
+          }
+          bf = __builtin_bit_cast(frag_t, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) acc[i][f] = M::mma(af[i], bf, acc[i][f]);
+      }
+    }
+  };
+
+  issue(0);
+  for (int it = 0; it < n_k; ++it) {
+    wait_dma();
+    __syncthreads();  // stage `it` is visible; everyone is done with the buffer stage it + 1 goes to
+    issue(it + 1);
+    compute(it);
+  }
+  wait_dma();
+  tile_epilogue<NFR, ACT>(a, t, acc, lds);
+}
+
+template <int XDT, int BM, int ACT, bool WKC>
+__global__ __launch_bounds__(256, 1) void mm_x16_w16_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr int MF = BM <= 32 ? 1 : BM / 32;
+  Tile t;
+  if (!locate_tile<BM, 0>(a, grid_n, grid_total, 1, t)) return;
+  const int nfr = (t.rows + 31) / 32;
+#define TAMD_CASE(n)                                                            \
+  case n:                                                                       \
+    if constexpr (n <= MF) run_tile_w16<XDT, n, 32 * MF, ACT, WKC>(a, t, lds);  \
+    break;
+  switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) }
+#undef TAMD_CASE
+}
+
+template <int XDT, int BM, int ACT, bool WKC>
+int launch_w16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  constexpr int MF = BM <= 32 ? 1 : BM / 32;
+  constexpr int LDS_ROWS = 32 * MF;
+  constexpr int PIPE = 2 * LDS_ROWS * A_ROW_BYTES + 2 * W16_STAGE;
+  constexpr int OUT_BYTES = LDS_ROWS * 256 * 2;
+  const int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
+  const int64_t total = (int64_t)grid_m * grid_n;
+  if (total <= 0) return 0;
+  const int64_t launch = ((total + 7) / 8) * 8;
+  if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+  auto kern = mm_x16_w16_kernel<XDT, BM, ACT, WKC>;
+  hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  kern<<<dim3((unsigned)launch), 256, PIPE > OUT_BYTES ? PIPE : OUT_BYTES, st>>>(a, grid_n, total);
+  return launch_status();
+}
+
+// 16-bit activations x 16-bit weights of the same type.  Returns TAMD_E_UNSUPPORTED / _ALIGNMENT for layouts
+// the kernel does not cover.
+template <int XDT>
+int dispatch_w16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  const bool kc = a.w_stride_k == 1, nc = a.w_stride_n == 1;
+  if (!kc && !nc) return TAMD_E_UNSUPPORTED;
+  if (a.K % 8 != 0) return TAMD_E_UNSUPPORTED;  // whole 16-byte chunks along K
+  if (!kc && a.N % 8 != 0) return TAMD_E_UNSUPPORTED;  // whole 16-byte chunks along N
+  const int64_t pitch = kc ? a.w_stride_n : a.w_stride_k;
+  if (!aligned(a.w, 16) || (pitch * 2) % 16 != 0 || (a.w_stride_e * 2) % 16 != 0) return TAMD_E_ALIGNMENT;
+  if (!aligned(a.x, 16) || (a.x_stride_m * 2) % 16 != 0 || (a.x_stride_z * 2) % 16 != 0) return TAMD_E_ALIGNMENT;
+  const int64_t x_rows = a.x_rows > 0 ? a.x_rows : a.M;
+  const int64_t w_span = (kc ? (int64_t)a.N * a.w_stride_n : (int64_t)a.K * a.w_stride_k) * 2;
+  if (x_rows * a.x_stride_m * 2 >= (int64_t)0x7FFFFF00 || w_span >= (int64_t)0x7FFFFF00) return TAMD_E_UNSUPPORTED;
+  const bool sw = a.activation == TAMD_ACT_SWIGLU;
+#define TAMD_W16(BMV)                                                                                           \
+  case BMV:                                                                                                     \
+    if (kc) return sw ? launch_w16<XDT, BMV, TAMD_ACT_SWIGLU, true>(a, grid_m, st)                               \
+                      : launch_w16<XDT, BMV, TAMD_ACT_NONE, true>(a, grid_m, st);                                 \
+    return sw ? launch_w16<XDT, BMV, TAMD_ACT_SWIGLU, false>(a, grid_m, st)                                      \
+              : launch_w16<XDT, BMV, TAMD_ACT_NONE, false>(a, grid_m, st);
+  switch (block_m) {
+    TAMD_W16(16) TAMD_W16(32) TAMD_W16(64) TAMD_W16(128)
+    default: return TAMD_E_UNSUPPORTED;
+  }
+#undef TAMD_W16
+}
+
+}  // namespace tamd

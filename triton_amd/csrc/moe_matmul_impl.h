@@ -187,6 +187,131 @@ TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
 constexpr int A_ROW_BYTES = 128;       // LDS bytes per activation row per stage (64 K of 16-bit, 128 K of fp8)
 constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K of fp4)
 
+// Epilogue of one output tile (shared by every tiled kernel).  The accumulators hold, for fragment
+// (i, f), element j: row 32i + 8(j/4) + 4h + j%4, column t.n0 + wave*64 + c32*NF + f.
+template <int NFR, int ACT>
+TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
+  const int tid = threadIdx.x;
+  const int wave = tid / kWave, lane = tid % kWave;
+  const int c32 = lane % 32, h = lane / 32;
+  const int N = a.N;
+  const int col0 = t.n0 + wave * 64 + c32 * NF;
+  // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
+  // column col0 + f.  16-bit outputs are staged through LDS (the K stages are dead by now) so
+  // that the global stores are 16 bytes per lane and whole rows of the tile are contiguous.
+  float flex = 1.0f;
+  if (a.x_scale) flex *= *a.x_scale;
+  if (a.w_scale) flex *= *a.w_scale;
+  float bias[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f)
+    bias[f] = (a.bias && col0 + f < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col0 + f)
+                                       : 0.f;
+  constexpr int NO = ACT == TAMD_ACT_SWIGLU ? NF / 2 : NF;  // outputs per lane per row
+  constexpr int OUT_COLS = 128 * NO;                        // output columns of the tile
+  const int n_out = ACT == TAMD_ACT_SWIGLU ? N / 2 : N;
+  const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
+  const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
+  const bool has_limit = a.act_has_limit != 0;
+  const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
+  const bool staged = osz < 4;
+  // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
+  const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
+  const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
+  const float out_max = max_finite_of(a.y_dtype);
+  uint32_t amax = 0;
+  auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
+    return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v)
+                                  : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
+  };
+  uint8_t *ob = lds;  // [rows][OUT_COLS] outputs of osz bytes
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < NFR; ++i) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
+      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
+      const float beta = a.betas ? a.betas[erow] : 1.0f;
+      const float gamma = a.gammas ? a.gammas[erow] : 1.0f;
+      float v[NF];
+#pragma unroll
+      for (int f = 0; f < NF; ++f) v[f] = (acc[i][f][j] * flex + bias[f] * beta) * a.out_alpha;
+      float o[NO];
+      if constexpr (ACT == TAMD_ACT_SWIGLU) {
+        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit) * gamma;
+      } else {
+#pragma unroll
+        for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
+      }
+      if (a.y_actual_scale && r < t.rows) {
+#pragma unroll
+        for (int p = 0; p < NO; ++p)
+          if (out_col0 + p < n_out) amax = absmax_bits(amax, o[p]);
+      }
+#pragma unroll
+      for (int p = 0; p < NO; ++p) {
+        o[p] *= inv_expected;
+        if (clamp_out) o[p] = __builtin_fminf(__builtin_fmaxf(o[p], -out_max), out_max);
+      }
+      if (staged) {
+        uint8_t *dstl = ob + (r * OUT_COLS + wave * 32 * NO + c32 * NO) * osz;
+        if (osz == 2) {
+          if constexpr (NO == 2) *(uint32_t *)dstl = narrow(o[0]) | (narrow(o[NO - 1]) << 16);
+          else *(uint16_t *)dstl = (uint16_t)narrow(o[0]);
+        } else {
+          if constexpr (NO == 2) *(uint16_t *)dstl = (uint16_t)(narrow(o[0]) | (narrow(o[NO - 1]) << 8));
+          else *dstl = (uint8_t)narrow(o[0]);
+        }
+      } else if (r < t.rows) {
+        int64_t dst = t.start_m + t.off_m + r;
+        if (a.scatter_indx) dst = a.scatter_indx[dst];
+        if (dst >= 0) {
+          const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
+#pragma unroll
+          for (int p = 0; p < NO; ++p)
+            if (out_col0 + p < n_out) ((float *)a.y)[base + out_col0 + p] = o[p];
+        }
+      }
+    }
+  }
+  if (a.y_actual_scale) {
+    // wave maximum, then one atomic per wave; positive floats order like their bit patterns
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
+      amax = other > amax ? other : amax;
+    }
+    if (lane == 0) {
+      amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
+      const float sc = __builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f);
+      atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(sc));
+    }
+  }
+  if (staged) {
+    __syncthreads();
+    const int epc = 16 / osz;                 // outputs per 16-byte chunk
+    const int cpr = OUT_COLS / epc;           // chunks per tile row
+    const int n_chunks = t.rows * cpr;
+    for (int id = tid; id < n_chunks; id += 256) {
+      const int r = id / cpr, c = (id - r * cpr) * epc;
+      int64_t dst = t.start_m + t.off_m + r;
+      if (a.scatter_indx) dst = a.scatter_indx[dst];
+      if (dst < 0) continue;
+      const int gcol = tile_out0 + c;
+      if (gcol >= n_out) continue;
+      uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * osz;
+      const uint8_t *sp = ob + (r * OUT_COLS + c) * osz;
+      if (gcol + epc <= n_out && ((uintptr_t)yp & 15) == 0) {
+        *(uint4 *)yp = *(const uint4 *)sp;
+      } else {
+        const int n_b = (n_out - gcol < epc ? n_out - gcol : epc) * osz;
+        for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
+      }
+    }
+  }
+}
+
 // One output tile with NFR (compile time) active 32-row fragments.
 // LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | e8m0 scales of the tile].
 //
@@ -401,120 +526,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   wait_dma();
 
-  // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
-  // column col0 + f.  16-bit outputs are staged through LDS (the K stages are dead by now) so
-  // that the global stores are 16 bytes per lane and whole rows of the tile are contiguous.
-  float flex = 1.0f;
-  if (a.x_scale) flex *= *a.x_scale;
-  if (a.w_scale) flex *= *a.w_scale;
-  float bias[NF];
-#pragma unroll
-  for (int f = 0; f < NF; ++f)
-    bias[f] = (a.bias && col0 + f < N) ? load_any_f32(a.bias, a.bias_dtype, (int64_t)t.expert * a.bias_stride_e + col0 + f)
-                                       : 0.f;
-  constexpr int NO = ACT == TAMD_ACT_SWIGLU ? NF / 2 : NF;  // outputs per lane per row
-  constexpr int OUT_COLS = 128 * NO;                        // output columns of the tile
-  const int n_out = ACT == TAMD_ACT_SWIGLU ? N / 2 : N;
-  const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
-  const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
-  const bool has_limit = a.act_has_limit != 0;
-  const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
-  const bool staged = osz < 4;
-  // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
-  const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
-  const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
-  const float out_max = max_finite_of(a.y_dtype);
-  uint32_t amax = 0;
-  auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
-    return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v)
-                                  : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
-  };
-  uint8_t *ob = lds;  // [rows][OUT_COLS] outputs of osz bytes
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < NFR; ++i) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
-      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
-      const float beta = a.betas ? a.betas[erow] : 1.0f;
-      const float gamma = a.gammas ? a.gammas[erow] : 1.0f;
-      float v[NF];
-#pragma unroll
-      for (int f = 0; f < NF; ++f) v[f] = (acc[i][f][j] * flex + bias[f] * beta) * a.out_alpha;
-      float o[NO];
-      if constexpr (ACT == TAMD_ACT_SWIGLU) {
-        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit) * gamma;
-      } else {
-#pragma unroll
-        for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
-      }
-      if (a.y_actual_scale && r < t.rows) {
-#pragma unroll
-        for (int p = 0; p < NO; ++p)
-          if (out_col0 + p < n_out) amax = absmax_bits(amax, o[p]);
-      }
-#pragma unroll
-      for (int p = 0; p < NO; ++p) {
-        o[p] *= inv_expected;
-        if (clamp_out) o[p] = __builtin_fminf(__builtin_fmaxf(o[p], -out_max), out_max);
-      }
-      if (staged) {
-        uint8_t *dstl = ob + (r * OUT_COLS + wave * 32 * NO + c32 * NO) * osz;
-        if (osz == 2) {
-          if constexpr (NO == 2) *(uint32_t *)dstl = narrow(o[0]) | (narrow(o[NO - 1]) << 16);
-          else *(uint16_t *)dstl = (uint16_t)narrow(o[0]);
-        } else {
-          if constexpr (NO == 2) *(uint16_t *)dstl = (uint16_t)(narrow(o[0]) | (narrow(o[NO - 1]) << 8));
-          else *dstl = (uint8_t)narrow(o[0]);
-        }
-      } else if (r < t.rows) {
-        int64_t dst = t.start_m + t.off_m + r;
-        if (a.scatter_indx) dst = a.scatter_indx[dst];
-        if (dst >= 0) {
-          const int64_t base = (int64_t)t.z * a.y_stride_z + dst * a.y_stride_m;
-#pragma unroll
-          for (int p = 0; p < NO; ++p)
-            if (out_col0 + p < n_out) ((float *)a.y)[base + out_col0 + p] = o[p];
-        }
-      }
-    }
-  }
-  if (a.y_actual_scale) {
-    // wave maximum, then one atomic per wave; positive floats order like their bit patterns
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
-      amax = other > amax ? other : amax;
-    }
-    if (lane == 0) {
-      amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
-      const float sc = __builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f);
-      atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(sc));
-    }
-  }
-  if (staged) {
-    __syncthreads();
-    const int epc = 16 / osz;                 // outputs per 16-byte chunk
-    const int cpr = OUT_COLS / epc;           // chunks per tile row
-    const int n_chunks = t.rows * cpr;
-    for (int id = tid; id < n_chunks; id += 256) {
-      const int r = id / cpr, c = (id - r * cpr) * epc;
-      int64_t dst = t.start_m + t.off_m + r;
-      if (a.scatter_indx) dst = a.scatter_indx[dst];
-      if (dst < 0) continue;
-      const int gcol = tile_out0 + c;
-      if (gcol >= n_out) continue;
-      uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * osz;
-      const uint8_t *sp = ob + (r * OUT_COLS + c) * osz;
-      if (gcol + epc <= n_out && ((uintptr_t)yp & 15) == 0) {
-        *(uint4 *)yp = *(const uint4 *)sp;
-      } else {
-        const int n_b = (n_out - gcol < epc ? n_out - gcol : epc) * osz;
-        for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
-      }
-    }
-  }
+  tile_epilogue<NFR, ACT>(a, t, acc, lds);
 }
 
 // Row fragments a workgroup can hold: a 128-row block of 16-bit activations also takes a remainder of
