@@ -157,7 +157,9 @@ typedef struct tamd_matmul_args {
   int x_dtype; /* TAMD_BF16 / TAMD_F16 / TAMD_FP8_E4M3 */
   int64_t x_stride_m;
   const float *x_scale; /* per-tensor flex scale (device scalar) or NULL */
-  /* weights: n_experts x [K, N]; MXFP4: packed bytes, K/2 bytes contiguous per column */
+  /* weights: n_experts x [K, N]; MXFP4: packed bytes, K/2 bytes contiguous per column.  TAMD_BF16 / TAMD_F16
+   * weights must have the activations' type, unit stride along K or along N, and K % 8 == 0 (N % 8 == 0 too when
+   * N is the contiguous axis) */
   const void *w;
   int w_dtype; /* TAMD_MXFP4 / TAMD_BF16 / TAMD_F16 */
   int64_t w_stride_e, w_stride_k, w_stride_n; /* in storage elements (bytes for MXFP4) */
