@@ -86,6 +86,15 @@ def make_weights(E, K, N, device, seed=0):
     return vals, scales
 
 
+def scales_for_matmul(scales, layout):
+    """The weight scales in the encoding asked for on the command line."""
+    if layout == "strided":
+        return scales
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
+    return convert_layout(wrap_torch_tensor(scales), CDNA4MXScaleLayout())
+
+
 def algorithmic_bytes(col_sum, T, k, K, N, act):
     """x rows read + y rows written + (codes + scales + bias) of the experts that have rows."""
     rows = T * k
@@ -140,7 +149,8 @@ def run_fc2(args, cfg):
     del x0
     logits, bias = logits_cpu.to(dev), bias_cpu.to(dev)
     vals, scales = make_weights(E, K, N, dev)
-    pc = PrecisionConfig(b_mx_scale=scales, b_microblock_size=32, out_dtype=torch.bfloat16,
+    pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32,
+                         out_dtype=torch.bfloat16,
                          flex_ctx=FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale)))
     y_buf = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
     constraints = {"block_m": args.block_m} if args.block_m else {}
@@ -205,7 +215,7 @@ def run_fc2(args, cfg):
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: routing + matmul_ogs(fp8 rows, grouped GEMM, bias, gate weights, scatter) + "
                                f"top-{k} combine, T={T}, hidden={K}, experts={E}, W2 mxfp4 [{E},{K},{N}]",
-                   "rows": rows, "active_experts": n_active},
+                   "rows": rows, "active_experts": n_active, "scale_layout": args.scale_layout},
         "tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
         "roofline": roof, "cpu_baseline": cpu,
         "parity": {"routing_bit_exact": routing_ok, "combine_bit_exact": combine_ok, "gemm_sample_within_1e-2": gemm_ok},
@@ -220,6 +230,9 @@ def main():
     ap.add_argument("--workload", default="fc1_prefill", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-experts", type=int, default=8, help="experts in the CPU baseline sample (0 = skip)")
     ap.add_argument("--block-m", type=int, default=0)
+    ap.add_argument("--scale-layout", default="strided", choices=["strided", "cdna4"],
+                    help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
+                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout()))")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (experts would shard across GPUs, "
@@ -252,7 +265,7 @@ def main():
     bias_cpu = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
     logits, x, bias = logits_cpu.to(dev), x_cpu.to(dev), bias_cpu.to(dev)
     vals, scales = make_weights(E, K, N, dev)
-    pc = PrecisionConfig(b_mx_scale=scales, b_microblock_size=32)
+    pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
     fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if act else None
     constraints = {"block_m": args.block_m} if args.block_m else {}
 
@@ -323,7 +336,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x mxfp4 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.workload}: routing + matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, "
                                f"hidden={K}, experts={E}, top-{k}, W1 mxfp4 [{E},{K},{N}]",
-                   "rows": rows, "active_experts": n_active},
+                   "rows": rows, "active_experts": n_active, "scale_layout": args.scale_layout},
         "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
         "matmul_kernel_tflops": round(tflops_kernel, 2),
         "roofline": roof,

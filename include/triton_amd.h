@@ -41,6 +41,10 @@ extern "C" {
 #define TAMD_FP8_E5M2 4
 #define TAMD_MXFP4 5    /* two e2m1 codes per byte, even index in the low nibble */
 
+/* encodings of the weight scales (tamd_matmul_args.w_mx_layout) */
+#define TAMD_SCALE_STRIDED 0
+#define TAMD_SCALE_CDNA4 1
+
 /* dequant-scale rounding of downcast_to_mxfp (numerics_details/mxfp.py:17-22) */
 #define TAMD_ROUND_UP 0
 #define TAMD_ROUND_DOWN 1
@@ -164,7 +168,7 @@ typedef struct tamd_matmul_args {
   int w_dtype; /* TAMD_MXFP4 / TAMD_BF16 / TAMD_F16 */
   int64_t w_stride_e, w_stride_k, w_stride_n; /* in storage elements (bytes for MXFP4) */
   const float *w_scale;                       /* per-tensor flex scale or NULL */
-  const uint8_t *w_mx_scale;                  /* e8m0 [E, K/32, N] or NULL */
+  const uint8_t *w_mx_scale;                  /* e8m0 [E, K/32, N] or NULL; see w_mx_layout */
   int64_t w_mx_stride_e, w_mx_stride_k, w_mx_stride_n;
   /* bias [E, N] (unit stride along N) or NULL */
   const void *bias;
@@ -208,6 +212,10 @@ typedef struct tamd_matmul_args {
   const float *y_expected_scale;
   float *y_actual_scale;
   int y_saturate_inf;
+  /* encoding of w_mx_scale: TAMD_SCALE_STRIDED (strides above) or TAMD_SCALE_CDNA4, the pre-shuffled storage of
+   * tensor_details/layout_details/cdna4_scale.py:32-68 (per expert: ceil(N/32) blocks of ceil(K/256)*8*32 bytes,
+   * 16-byte aligned; only w_mx_stride_e is used) */
+  int w_mx_layout;
 } tamd_matmul_args;
 
 int tamd_matmul(const tamd_matmul_args *args, void *stream);

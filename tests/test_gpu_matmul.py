@@ -461,3 +461,83 @@ def test_ragged_16bit_weights(block_m, act, device):
     ref = MR.matmul_ref(x, w, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, gammas=gammas,
                         fused_swiglu=(1.702, 7.0) if act else None)
     check(out, ref)
+
+
+# ---------------------------------------------------------------------------- pre-shuffled (CDNA4) weight scales
+
+
+def preshuffle(s):
+    """Scales as downcast_to_mxfp returns them -> the CDNA4 scale layout, checked against the oracle's bytes."""
+    import numpy as np
+    from oracle import layout_ref as LR
+    from triton_amd.tensor import convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
+    t = convert_layout(wrap_torch_tensor(s), CDNA4MXScaleLayout())
+    d = t.storage.data
+    flat = d.transpose(-1, -2).reshape(d.shape[0], d.shape[1] * d.shape[2]).cpu().numpy()
+    assert np.array_equal(flat, LR.cdna4_swizzle_ref(s.cpu().contiguous().numpy()))
+    return t
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 2048, 4096), (16, 64, 64), (33, 96, 208), (130, 192, 528), (1, 32, 16),
+                                   (70, 2880, 5760 // 8)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_dense_with_preshuffled_scales(M, K, N, fp8, device):
+    """The same kernel, same arithmetic: results must equal the strided-scale ones bit for bit, and match the oracle."""
+    torch.manual_seed(0)
+    w = torch.randn(K, N) * 0.02
+    bias = (torch.randn(N) * 0.01).to(torch.bfloat16)
+    v, s, rv, rs = quantize_w(w, device)
+    if fp8:
+        x, x_scale = to_fp8(torch.randn(M, K))
+        flex = FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale.to(device)))
+        mk = lambda sc: PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, flex_ctx=flex, out_dtype=torch.bfloat16)
+        ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs, a_flex_scale=x_scale).to(torch.bfloat16)
+    else:
+        x = torch.randn(M, K).to(torch.bfloat16)
+        mk = lambda sc: PrecisionConfig(b_mx_scale=sc, b_microblock_size=32)
+        ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs)
+    out_s = matmul(x.to(device), v, bias.to(device), precision_config=mk(s))
+    out_p = matmul(x.to(device), v, bias.to(device), precision_config=mk(preshuffle(s)))
+    assert torch.equal(out_p, out_s)
+    check(out_p, ref)
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 32, 128])
+@pytest.mark.parametrize("K,N", [(320, 400), (2880, 608), (4096, 96)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_ragged_with_preshuffled_scales(block_m, K, N, fp8, device):
+    """Ragged, gather + scatter + gate weights + SwiGLU; block_m 16 with N % 16 == 0 runs the streaming kernel,
+    whose units are halves of the 32-column scale blocks."""
+    torch.manual_seed(1)
+    E = 7
+    sizes = torch.tensor([3, 0, 1, 16, 5, 140, 2], dtype=torch.int32)
+    M = int(sizes.sum())
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    gather = torch.randint(0, M + 5, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::7] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    kw = dict(slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs, gammas=gammas,
+              fused_swiglu=(1.702, 7.0))
+    if fp8:
+        x, x_scale = to_fp8(torch.randn(M + 5, K))
+        flex = FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale.to(device)))
+        mk = lambda sc: PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, flex_ctx=flex, out_dtype=torch.bfloat16)
+        ref = MR.matmul_ref(x, rv, bias, a_flex_scale=x_scale, **kw).to(torch.bfloat16)
+    else:
+        x = torch.randn(M + 5, K).to(torch.bfloat16)
+        mk = lambda sc: PrecisionConfig(b_mx_scale=sc, b_microblock_size=32)
+        ref = MR.matmul_ref(x, rv, bias, **kw)
+    outs = []
+    for sc in (s, preshuffle(s)):
+        out_init = torch.zeros((M, N // 2), dtype=torch.bfloat16, device=device)
+        with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+            outs.append(matmul(x.to(device), v, bias.to(device), md, gather_indx=gather.to(device),
+                               scatter_indx=scatter.to(device), precision_config=mk(sc), gammas=gammas.to(device),
+                               fused_activation=swiglu_act(1.702, 7.0), c=out_init))
+    assert torch.equal(outs[1], outs[0])
+    check(outs[1], ref)

@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("TAMD_LIB") or os.path.join(_HERE, "libtriton_amd.so")
 # element type codes (include/triton_amd.h)
 F32, F16, BF16, FP8_E4M3, FP8_E5M2, MXFP4 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_SWIGLU = 0, 1
+SCALE_STRIDED, SCALE_CDNA4 = 0, 1
 E_INVALID, E_UNSUPPORTED, E_ALIGNMENT = -1, -2, -3
 
 _TORCH_CODE = {
@@ -50,6 +51,7 @@ class MatmulArgs(C.Structure):
         ("activation", C.c_int), ("act_alpha", C.c_float), ("act_limit", C.c_float), ("act_has_limit", C.c_int),
         ("force_variant", C.c_int), ("x_rows", C.c_int64),
         ("y_expected_scale", C.c_void_p), ("y_actual_scale", C.c_void_p), ("y_saturate_inf", C.c_int),
+        ("w_mx_layout", C.c_int),
     ]
 
 

@@ -36,13 +36,16 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     if (!a.w_mx_scale) return TAMD_E_INVALID;
     if (a.K % 32 != 0) return TAMD_E_INVALID;
     // weights / scales must be contiguous along K ("column-major" mxfp weights)
-    if (a.w_stride_k != 1 || a.w_mx_stride_k != 1) return TAMD_E_UNSUPPORTED;
+    const bool cdna4_sc = a.w_mx_layout == TAMD_SCALE_CDNA4;
+    if (a.w_mx_layout != TAMD_SCALE_STRIDED && !cdna4_sc) return TAMD_E_INVALID;
+    if (a.w_stride_k != 1 || (!cdna4_sc && a.w_mx_stride_k != 1)) return TAMD_E_UNSUPPORTED;
+    if (cdna4_sc && (!aligned(a.w_mx_scale, 16) || a.w_mx_stride_e % 16 != 0)) return TAMD_E_ALIGNMENT;
     if (!aligned(a.w, 16) || a.w_stride_n % 16 != 0 || a.w_stride_e % 16 != 0) return TAMD_E_ALIGNMENT;
     if (!aligned(a.x, 16) || (a.x_stride_m * esz) % 16 != 0 || (a.x_stride_z * esz) % 16 != 0) return TAMD_E_ALIGNMENT;
     // 32-bit buffer offsets: one batch of activations and one expert's weights must each span < 2 GiB
     const int64_t x_rows = a.x_rows > 0 ? a.x_rows : a.M;
     if (x_rows * a.x_stride_m * esz >= (int64_t)0x7FFFFF00 || (int64_t)a.N * a.w_stride_n >= (int64_t)0x7FFFFF00 ||
-        (int64_t)a.N * a.w_mx_stride_n >= (int64_t)0x7FFFFF00)
+        (int64_t)a.N * (cdna4_sc ? (int64_t)(a.K / 32 + 7) : a.w_mx_stride_n) >= (int64_t)0x7FFFFF00)
       return TAMD_E_UNSUPPORTED;
     int block_m, grid_m;
     if (ragged) {

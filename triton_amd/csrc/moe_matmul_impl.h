@@ -345,16 +345,23 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const uint8_t *bbuf = lds + 2 * A_STAGE + wave * 4096;
   uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES;
 
-  // ---- scales of the whole tile, once: 256 columns x G bytes, contiguous in memory
+  // ---- scales of the whole tile, once.  Strided: 256 columns x G bytes, contiguous in memory.  CDNA4
+  // pre-shuffle: the tile's 8 blocks of 32 columns are contiguous too (KSP*32 bytes each); byte
+  // 256*(k/8) + 64*(k%4) + 4*(n%16) + 2*((k%8)/4) + (n%32)/16 of a block is the scale of (group k, column n).
+  const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
+  const int KSP = (G + 7) / 8 * 8;
   const int tile_cols = N - t.n0 < BLOCK_N ? N - t.n0 : BLOCK_N;
+  const int64_t sc_tile_off = cdna4 ? (int64_t)(t.n0 / 32) * KSP * 32 : (int64_t)t.n0 * G;
   if constexpr (SC_LDS) {
-    const uint8_t *sc_src = s_base + (int64_t)t.n0 * G;
-    if ((((uintptr_t)sc_src) & 15) == 0 && (N * G) % 16 == 0) {
+    const uint8_t *sc_src = s_base + sc_tile_off;
+    const int sc_tile_bytes = BLOCK_N * (cdna4 ? KSP : G);
+    const int sc_avail = cdna4 ? ((N + 31) / 32 * 32 - t.n0) * KSP : (N - t.n0) * G;  // bytes up to the expert's end
+    if (cdna4 || ((((uintptr_t)sc_src) & 15) == 0 && (N * G) % 16 == 0)) {
       // by DMA, 1 KB per instruction: in flight together with the first activation / weight stages and
       // awaited with them at the first barrier of the K loop
-      const v4i_t rs = make_rsrc(sc_src, (uint32_t)((N - t.n0) * G));
+      const v4i_t rs = make_rsrc(sc_src, (uint32_t)sc_avail);
       const uint32_t lds_sc_addr = lds_base + 2 * A_STAGE + B_BYTES;
-      for (int i = wave; i * 1024 < BLOCK_N * G; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
+      for (int i = wave; i * 1024 < sc_tile_bytes; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
     } else {
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
                                                                         0x00020000);
@@ -363,6 +370,21 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
     }
   }
+  // offset of a column's scales inside the tile's image (LDS) or, without staging, from the expert's first scale
+  int sc_col_off[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int tc = wave * 64 + c32 * NF + f;  // tile column
+    if constexpr (SC_LDS) {
+      sc_col_off[f] = cdna4 ? (tc / 32) * KSP * 32 + (tc % 16) * 4 + (tc % 32) / 16 : tc * G;
+    } else {
+      const int col = t.n0 + tc < N ? t.n0 + tc : N - 1;
+      sc_col_off[f] = cdna4 ? (col / 32) * KSP * 32 + (col % 16) * 4 + (col % 32) / 16 : 0;  // strided: 64-bit below
+    }
+  }
+
+  const int sc_lane_off[2] = {h * (cdna4 ? 64 : 1), (2 + h) * (cdna4 ? 64 : 1)};  // the (2q + h) part of a group's offset
+  const int sc_clamp = cdna4 ? 0x7FFFFFFF : G - 1;
 
   // ---- activation DMA: one instruction per 32-row fragment, lane -> (row 8w + lane/8, slot lane%8)
   const int a_rin = wave * 8 + lane / 8;
@@ -427,10 +449,17 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       for (int q = 0; q < 2; ++q) {
         const int pos = f * 32 + c32;
         raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
-        const int kg = sup * 4 + 2 * q + h;
+        // group kg = 4*sup + 2q + h of this lane's column.  Strided: byte kg, kept inside the column's G bytes
+        // (groups past the end of K meet zero codes and zero activations; their scale only has to be some finite
+        // value of this column).  Pre-shuffled: byte 256*(kg/8) + 64*(kg%4) + 2*((kg%8)/4); the padding up to a
+        // multiple of 8 groups is stored (zeros), so nothing is clamped.
+        const int sup_off = cdna4 ? (sup >> 1) * 256 + (sup & 1) * 2 : sup * 4;  // wave uniform
+        int kg_off = sup_off + sc_lane_off[q];
+        kg_off = kg_off < sc_clamp ? kg_off : sc_clamp;
         uint32_t sbyte;
-        if constexpr (SC_LDS) sbyte = lds_sc[(wave * 64 + c32 * NF + f) * G + (kg < G ? kg : G - 1)];
-        else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + (kg < G ? kg : G - 1)];
+        if constexpr (SC_LDS) sbyte = lds_sc[sc_col_off[f] + kg_off];
+        else if (cdna4) sbyte = s_base[sc_col_off[f] + kg_off];
+        else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + kg_off];
         if constexpr (FP8) scw[f] = q == 0 ? sbyte : (scw[f] | (sbyte << 8));
         else scf[f][q] = bits_to_f32(sbyte << 23);
       }
@@ -577,11 +606,12 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   if (total <= 0) return 0;
   int64_t launch = ((total + 7) / 8) * 8;
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-  // scales of a tile are staged in LDS when they are dense ([N][K/32]) and two workgroups still fit a CU
+  // scales of a tile are staged in LDS when they are dense ([N][K/32]) or pre-shuffled and two workgroups still fit a CU
   const int64_t G = a.K / 32;
-  const int64_t sc_bytes = (BLOCK_N * G + 1023) / 1024 * 1024;  // whole 1 KB copies
-  const bool dense_sc = a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
-                        aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0;
+  const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
+  const int64_t sc_bytes = (BLOCK_N * (cdna4 ? (G + 7) / 8 * 8 : G) + 1023) / 1024 * 1024;  // whole 1 KB copies
+  const bool dense_sc = cdna4 || (a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
+                                  aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0);
   const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;
   size_t lds_bytes = PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
   if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;

@@ -92,12 +92,13 @@ TAMD_DEVICE void dma16_at(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t
 template <int SS, int RING_>
 struct StreamShape {
   static constexpr int CODE_BYTES = 4 * SS * 1024;  // image of 16 columns' codes, padded to whole 1 KB copies
-  static constexpr int SC_BYTES = 2048;             // image of their scales (16 * K/32 <= 2048 bytes)
+  static constexpr int NSC = (SS + 1) / 2;          // 1 KB pieces of the scale image: 16 * K/32 bytes, or the whole
+  static constexpr int SC_BYTES = NSC * 1024;       // pre-shuffled block of 32 columns (ceil(K/256)*8 * 32 bytes)
   static constexpr int BIAS_BYTES = 256;            // 16 bias values, one dword each
   static constexpr int STAGE = CODE_BYTES + SC_BYTES + BIAS_BYTES;
   static constexpr int RED_BYTES = 2 * 4 * 1024;    // partial sums: 2 buffers x 4 waves x 16x16 floats
   static constexpr int RING = RING_;
-  static constexpr int DMA_PER_STAGE = 2 * SS + 2;  // most copies one wave has per stage
+  static constexpr int DMA_PER_STAGE = 2 * SS + NSC;  // most copies one wave has per stage
   static constexpr int LDS = RING * STAGE + RED_BYTES;
   static_assert(RING >= 2 && (RING - 1) * DMA_PER_STAGE < 64, "ring does not fit the vmcnt counter");
 };
@@ -291,13 +292,17 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       const uint32_t lin = (uint32_t)(half * NP + i) * 1024u + lane * 16u;
       w_voff[i] = lin < 16u * col_bytes ? (uint32_t)(half * NP) * 1024u + lane * 16u : kOob;  // piece i adds i*1024 itself
     }
-    uint32_t x_voff[2];
+    // scale image of a unit: its 16 * G bytes, or (pre-shuffled scales) the block of 32 columns it lies in
+    const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
+    const uint32_t sc_unit_bytes = cdna4 ? (uint32_t)((G + 7) / 8 * 8 * 32) : (uint32_t)(16 * G);
+    uint32_t x_voff[S::NSC];
     if (half == 0) {
 #pragma unroll
-      for (int q = 0; q < 2; ++q) x_voff[q] = q * 1024u + lane * 16u < (uint32_t)(16 * G) ? q * 1024u + lane * 16u : kOob;
+      for (int q = 0; q < S::NSC; ++q) x_voff[q] = q * 1024u + lane * 16u < sc_unit_bytes ? q * 1024u + lane * 16u : kOob;
     } else {
       x_voff[0] = (a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
-      x_voff[1] = kOob;
+#pragma unroll
+      for (int q = 1; q < S::NSC; ++q) x_voff[q] = kOob;
     }
     int i_blk = blk0 - 1, i_cg = cg0, i_left = total_stages;
     uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0;
@@ -310,7 +315,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         get_block(i_blk, b);
         const int e = __builtin_amdgcn_readfirstlane(b.expert);  // keeps the running offsets in scalar registers
         i_wbase = (uint32_t)((int64_t)e * a.w_stride_e) + (uint32_t)i_cg * 16u * col_bytes;
-        i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e) + (uint32_t)(i_cg * 16 * G);
+        i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e);
         i_bbase = (uint32_t)(((int64_t)e * a.bias_stride_e + i_cg * 16) * bias_esz);
       }
       const uint32_t sb = lds_base + slot * S::STAGE;
@@ -325,15 +330,16 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         if (i % 4 == 3) dma16_at<3072, false>(dw, m0v, w_voff[i], so);
       }
       if (half == 0) {
-        dma16(live ? rs : rs0, sb + S::CODE_BYTES, x_voff[0], i_sbase);
-        dma16(live ? rs : rs0, sb + S::CODE_BYTES + 1024, x_voff[1], i_sbase);
+        const uint32_t so = i_sbase + (cdna4 ? (uint32_t)(i_cg >> 1) : (uint32_t)i_cg) * sc_unit_bytes;
+#pragma unroll
+        for (int q = 0; q < S::NSC; ++q) dma16(live ? rs : rs0, sb + S::CODE_BYTES + q * 1024, x_voff[q], so);
       } else {
         const uint32_t dst = sb + S::CODE_BYTES + S::SC_BYTES;
         if (bias_esz == 4) dma4(live ? rb : rb0, dst, x_voff[0], i_bbase);
         else dma2(live ? rb : rb0, dst, x_voff[0], i_bbase);
       }
       ++i_cg, --i_left;
-      i_wbase += 16u * col_bytes, i_sbase += (uint32_t)(16 * G), i_bbase += (uint32_t)(16 * bias_esz);
+      i_wbase += 16u * col_bytes, i_bbase += (uint32_t)(16 * bias_esz);
     };
     // stage s lives in slot s % RING and is requested RING - 1 stages ahead
     int i_slot = 0;
@@ -345,7 +351,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
 #pragma unroll 1
     for (int s = 0; s < total_stages; ++s) {
       // copies complete in order: once at most RING - 2 stages' worth are outstanding, stage s has landed
-      if (half == 0) wait_vmcnt<(S::RING - 2) * (NP + 2)>();
+      if (half == 0) wait_vmcnt<(S::RING - 2) * (NP + S::NSC)>();
       else wait_vmcnt<(S::RING - 2) * (NP + 1)>();
       __syncthreads();  // publishes stage s; every wave is done with stage s - 1, whose slot is refilled now
       issue(i_slot);
@@ -356,6 +362,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
   } else {
     // =========================================================================== compute waves
     const int c16 = lane % 16, g = lane / 16;
+    const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
     const int kb = 4 * SS * wave;  // first e8m0 group of this wave's K slice
     frag_t areg[SS * 4];           // this wave's K slice of the block's rows, row c16
     int c_blk = blk0 - 1, c_cg = cg0;
@@ -386,7 +393,9 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       const int kg = kb + 4 * j + g;
       kvalid[j] = kg < G;
       b_loff[j] = (uint32_t)c16 * col_bytes + (kvalid[j] ? kg : 0) * 16;
-      s_loff[j] = (uint32_t)(S::CODE_BYTES + c16 * G + (kvalid[j] ? kg : 0));
+      const int kgv = kvalid[j] ? kg : 0;
+      s_loff[j] = (uint32_t)(S::CODE_BYTES +
+                             (cdna4 ? (kgv / 8) * 256 + (kgv % 4) * 64 + c16 * 4 + ((kgv % 8) / 4) * 2 : c16 * G + kgv));
     }
     int slot = 0;
 #pragma unroll 1
@@ -396,6 +405,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         if (c_cg == n_cg) c_cg = 0;
         load_block(++c_blk);
       }
+      const uint32_t sc_par = cdna4 ? (uint32_t)(c_cg & 1) : 0u;  // which 16 of the block's 32 columns
       ++c_cg;
       const uint8_t *img = lds + slot * S::STAGE;
       uint4 raw[SS];
@@ -403,7 +413,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
 #pragma unroll
       for (int j = 0; j < SS; ++j) {
         raw[j] = *(const uint4 *)(img + b_loff[j]);
-        sby[j] = img[s_loff[j]];
+        sby[j] = img[s_loff[j] + sc_par];
       }
       // four independent accumulation chains keep dependent MFMAs apart
       f32x4_t acc0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0, acc3 = acc0;
@@ -429,10 +439,12 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   const int64_t lim = 0x7FFFFF00;
   const int64_t G = a.K / 32;
   if (a.K > 4096 || a.K % 32 != 0) return false;
-  if (a.w_stride_k != 1 || a.w_stride_n != a.K / 2 || a.w_mx_stride_k != 1 || a.w_mx_stride_n != G) return false;
+  const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
+  if (a.w_stride_k != 1 || a.w_stride_n != a.K / 2) return false;
+  if (!cdna4 && (a.w_mx_stride_k != 1 || a.w_mx_stride_n != G)) return false;
   if (!aligned(a.w, 16) || a.w_stride_e % 16 != 0 || !aligned(a.w_mx_scale, 16) || a.w_mx_stride_e % 16 != 0) return false;
   if ((int64_t)a.n_experts * a.w_stride_e + (int64_t)a.N * a.w_stride_n >= lim) return false;
-  if ((int64_t)a.n_experts * a.w_mx_stride_e + (int64_t)a.N * G >= lim) return false;
+  if ((int64_t)a.n_experts * a.w_mx_stride_e + (int64_t)(a.N + 32) * (G + 8) >= lim) return false;
   if (a.bias && ((int64_t)a.n_experts * a.bias_stride_e + a.N) * 4 >= lim) return false;
   if (a.bias && !aligned(a.bias, a.bias_dtype == TAMD_F32 ? 4 : 2)) return false;
   if (a.N % 16 != 0) return false;  // whole 16-column groups only (their scale run is then a multiple of 16 bytes)
@@ -442,7 +454,7 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
 
 template <int XDT, int ACT, int SS>
 int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + 2048 + 256);
+  constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + (SS + 1) / 2 * 1024 + 256);
   constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
   const int n_cg = (a.N + 15) / 16;
   const int64_t upper = (int64_t)grid_m * n_cg;

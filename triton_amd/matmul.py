@@ -3,6 +3,7 @@ activation, gamma -> scatter (matmul.py:243-749 of the reference), over the
 gfx950 kernels.  Argument names, defaults and error behaviour follow the
 reference; combinations that are not built raise NotImplementedError."""
 import ctypes
+import math
 from dataclasses import dataclass
 from typing import Callable, Optional
 
@@ -15,6 +16,7 @@ from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_op
 from .numerics import InFlexData, OutFlexData
 from .specialize import FnSpecs
 from .tensor import FP4, RaggedTensorMetadata, Tensor, wrap_torch_tensor
+from .tensor_details.layout import CDNA4MXScaleLayout
 
 __all__ = ["matmul", "matmul_ogs", "PrecisionConfig", "FlexCtx", "FusedActivation", "Epilogue", "FnSpecs",
            "InFlexData", "OutFlexData", "InapplicableConstraint", "OptFlags", "scoped_opt_flags",
@@ -126,6 +128,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         assert precision_config.b_microblock_size is not None, \
             "precision_config.b_microblock_size is required when precision_config.b_mx_scale is set"
         assert precision_config.b_microblock_size == MXFP_BLOCK_SIZE, "Unsupported microscale block size"
+        b_scale_cdna4 = isinstance(b_scale, Tensor) and isinstance(b_scale.storage.layout, CDNA4MXScaleLayout)
+        b_scale_shape = list(b_scale.shape)
         b_scale = _data(b_scale)
         assert b_scale.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.dtype}"
     if isinstance(a, Tensor):
@@ -195,11 +199,22 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if b.dtype == FP4:
         assert b_scale is not None, "MXFP4 weights need precision_config.b_mx_scale"
         args.w_dtype = _lib.MXFP4
-        sd = b_scale if b_scale.ndim == 3 else b_scale[None]
-        assert tuple(sd.shape) == (wd.shape[0], K // MXFP_BLOCK_SIZE, N), \
-            f"b_mx_scale shape {tuple(sd.shape)} != {(wd.shape[0], K // MXFP_BLOCK_SIZE, N)}"
-        args.w_mx_scale = sd.data_ptr()
-        args.w_mx_stride_e, args.w_mx_stride_k, args.w_mx_stride_n = sd.stride()
+        want = [wd.shape[0], K // MXFP_BLOCK_SIZE, N]
+        if b_scale_cdna4:
+            # pre-shuffled storage [E, K_SCALE_pad * 32, N_pad / 32], block after block in memory
+            assert b_scale_shape[-2:] == want[-2:] and math.prod(b_scale_shape[:-2]) == want[0], \
+                f"b_mx_scale shape {b_scale_shape} != {want}"
+            assert list(b_scale.shape) == CDNA4MXScaleLayout().storage_shape(want) and \
+                (b_scale.numel() == 0 or (b_scale.stride(1) == 1 and b_scale.stride(2) == b_scale.shape[1])), \
+                "b_mx_scale storage does not match the CDNA4 scale layout"
+            args.w_mx_scale = b_scale.data_ptr()
+            args.w_mx_layout = _lib.SCALE_CDNA4
+            args.w_mx_stride_e, args.w_mx_stride_k, args.w_mx_stride_n = b_scale.stride(0), 0, 0
+        else:
+            sd = b_scale if b_scale.ndim == 3 else b_scale[None]
+            assert list(sd.shape) == want, f"b_mx_scale shape {tuple(sd.shape)} != {tuple(want)}"
+            args.w_mx_scale = sd.data_ptr()
+            args.w_mx_stride_e, args.w_mx_stride_k, args.w_mx_stride_n = sd.stride()
     else:
         args.w_dtype = _lib.dtype_code(w.dtype)
     args.w_stride_e, args.w_stride_k, args.w_stride_n = wd.stride()

@@ -10,7 +10,7 @@ from .tensor_details import bitmatrix as _bitmatrix
 from .tensor_details import ragged_tensor as _ragged
 from .tensor_details.dtype import (BF16, BIT, FP4, FP8_E4M3FN, FP8_E4M3FNUZ, FP8_E5M2, FP16, FP32, FP64, INT16,
                                    INT32, INT64, UINT8, DataType, FloatType, IntegerType)
-from .tensor_details.layout import Layout, StridedLayout
+from .tensor_details.layout import CDNA4MXScaleLayout, Layout, StridedLayout
 from .tensor_details.ragged_tensor import RaggedTensorMetadata
 from .tensor_details.bitmatrix import BitmatrixMetadata
 
@@ -134,9 +134,22 @@ def empty(shape, dtype, device, layout=None) -> Tensor:
 
 
 def convert_layout(tensor: Tensor, layout: Layout) -> Tensor:
-    """Re-packs `tensor` so that `layout.major_dim` is the contiguous (packed) axis."""
-    if not isinstance(layout, StridedLayout) or not isinstance(tensor.storage.layout, StridedLayout):
-        raise NotImplementedError("only strided layouts exist on gfx950")
+    """Re-encodes `tensor` in `layout`: another contiguous (packed) axis, or the CDNA4 scale pre-shuffle and back
+    (reference tensor.py:235-252).  Returns `tensor` itself when its storage already has that encoding."""
+    src = tensor.storage.layout
+    if isinstance(src, CDNA4MXScaleLayout) or isinstance(layout, CDNA4MXScaleLayout):
+        if src == layout:
+            return tensor
+        assert tensor.dtype != FP4, "the CDNA4 scale layout holds bytes"
+        data = tensor.storage.data
+        if isinstance(src, CDNA4MXScaleLayout):
+            data = src.make_transformation(tensor.shape).unswizzle_data(data)
+        if isinstance(layout, CDNA4MXScaleLayout):
+            data = layout.make_transformation(tensor.shape).swizzle_data(data)
+            return Tensor(Storage(data, layout), dtype=tensor.dtype, shape=list(tensor.shape))
+        return convert_layout(wrap_torch_tensor(data, dtype=tensor.dtype), layout)
+    if not isinstance(layout, StridedLayout) or not isinstance(src, StridedLayout):
+        raise NotImplementedError(f"layout {type(layout).__name__} does not exist on gfx950")
     rank = tensor.ndim
     if tensor.storage.layout.order(rank) == layout.order(rank):
         return tensor

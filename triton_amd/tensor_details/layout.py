@@ -1,7 +1,12 @@
-"""Storage layouts.  Only the strided layout (which axis is contiguous / packed)
-is needed on gfx950 for values; see tensor_details/layout_details/strided.py of
-the reference for the ordering rule reproduced by `StridedLayout.order`."""
+"""Storage layouts.  Values use the strided layout (which axis is contiguous / packed; see
+tensor_details/layout_details/strided.py of the reference for the ordering rule reproduced by
+`StridedLayout.order`).  Weight scales may also come pre-shuffled for CDNA4
+(`CDNA4MXScaleLayout`, reference tensor_details/layout_details/cdna4_scale.py:11-77), which is what
+`make_default_matmul_mxfp4_w_scale_layout` selects on this target (reference tensor_details/layout.py:43-54)."""
+import math
 from dataclasses import dataclass
+
+import torch
 
 
 @dataclass(frozen=True)
@@ -55,5 +60,73 @@ def make_default_matmul_mxfp4_w_layout(mx_axis: int, **_):
     return StridedLayout(-2)
 
 
+@dataclass(frozen=True)
+class CDNA4MXScaleLayoutTransformation:
+    """Pre-shuffle of e8m0 scales `[..., K/32, N]` for CDNA4 (reference cdna4_scale.py:32-77).
+
+    K/32 is padded to a multiple of 8 and N to a multiple of 32 (with zeros).  Columns are cut into blocks of 32;
+    a block's scales are one contiguous run of `K_SCALE_pad * 32` bytes in which the scale of group
+    `k = 8*k8 + 4*k2 + k4` of column `n = 32*nb + 16*n2 + n16` sits at byte
+
+        256*k8 + 64*k4 + 4*n16 + 2*k2 + n2
+
+    so that one dword holds, for one column pair (n16, n16 + 16), the groups k4 and k4 + 4: the four scale bytes a
+    lane of a 16-wide scaled MFMA selects from with op_sel.  Storage is `[B, K_SCALE_pad * 32, N_pad / 32]` with unit
+    stride along the middle axis, i.e. block after block in memory."""
+    shape: tuple
+    is_fp4: bool = False
+
+    def __post_init__(self):
+        assert not self.is_fp4, "scales are bytes"
+        *leading, k_scale, n = self.shape
+        object.__setattr__(self, "leading_shape", list(leading))
+        object.__setattr__(self, "B", math.prod(leading))
+        object.__setattr__(self, "K_SCALE", k_scale)
+        object.__setattr__(self, "N", n)
+        object.__setattr__(self, "K_SCALE_pad", -(-k_scale // 8) * 8)
+        object.__setattr__(self, "N_pad", -(-n // 32) * 32)
+
+    @property
+    def storage_shape(self):
+        return [self.B, self.K_SCALE_pad * 32, self.N_pad // 32]
+
+    def swizzle_data(self, data):
+        """`data`: `[..., K_SCALE, N]`, any strides."""
+        B, kp, npad = self.B, self.K_SCALE_pad, self.N_pad
+        x = data.reshape(B, self.K_SCALE, self.N)
+        x = torch.nn.functional.pad(x, (0, npad - self.N, 0, kp - self.K_SCALE))
+        x = x.reshape(B, kp // 8, 2, 4, npad // 32, 2, 16)  # b, k8, k2, k4, nb, n2, n16
+        x = x.permute(0, 4, 1, 3, 6, 2, 5).contiguous()      # b, nb, k8, k4, n16, k2, n2
+        out = x.reshape(B, npad // 32, kp * 32).transpose(-1, -2)
+        assert list(out.shape) == self.storage_shape
+        return out
+
+    def unswizzle_data(self, data):
+        """Back to a contiguous `[..., K_SCALE, N]`."""
+        B, kp, npad = self.B, self.K_SCALE_pad, self.N_pad
+        x = data.transpose(-1, -2).reshape(B, npad // 32, kp // 8, 4, 16, 2, 2)  # b, nb, k8, k4, n16, k2, n2
+        x = x.permute(0, 2, 5, 3, 1, 6, 4)                                        # b, k8, k2, k4, nb, n2, n16
+        x = x.reshape(B, kp, npad)[:, :self.K_SCALE, :self.N]
+        return x.reshape(*self.leading_shape, self.K_SCALE, self.N).contiguous()
+
+
+@dataclass(frozen=True)
+class CDNA4MXScaleLayout(Layout):
+
+    @property
+    def name(self):
+        return "CDNA4_SCALE"
+
+    def make_transformation(self, shape, is_fp4: bool = False):
+        return CDNA4MXScaleLayoutTransformation(tuple(shape), is_fp4)
+
+    def storage_shape(self, shape, is_fp4: bool = False):
+        return self.make_transformation(shape, is_fp4).storage_shape
+
+    def swizzle_block_shape(self, block_shape):
+        scale_k, n = block_shape[-2], block_shape[-1]
+        return list(block_shape[:-2]) + [n // 32, scale_k * 32]
+
+
 def make_default_matmul_mxfp4_w_scale_layout(mx_axis: int, num_warps: int = 8):
-    return StridedLayout(-2)
+    return CDNA4MXScaleLayout()
