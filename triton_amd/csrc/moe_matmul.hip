@@ -15,8 +15,9 @@ using namespace tamd;
 
 extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
   if (!args) return TAMD_E_INVALID;
-  const tamd_matmul_args &a = *args;
+  tamd_matmul_args a = *args;
   if (a.M < 0 || a.N < 0 || a.K < 0 || a.n_experts < 1) return TAMD_E_INVALID;
+  if (a.n_experts == 1) a.w_stride_e = a.w_mx_stride_e = a.bias_stride_e = 0;  // never used; keeps the alignment checks honest
   if (a.M == 0 || a.N == 0) return 0;
   if (!a.x || !a.w || !a.y) return TAMD_E_INVALID;
   if (a.activation != TAMD_ACT_NONE && a.activation != TAMD_ACT_SWIGLU) return TAMD_E_INVALID;
@@ -52,8 +53,9 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
       block_m = a.block_m;
       grid_m = a.grid_m;
     } else {
-      block_m = a.force_variant ? a.force_variant : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128);
-      grid_m = ((a.M + block_m - 1) / block_m) * a.n_experts;
+      // 0: the dispatcher chooses (it knows which kernels apply)
+      block_m = a.force_variant;
+      grid_m = block_m ? ((a.M + block_m - 1) / block_m) * a.n_experts : 0;
     }
     if (a.x_dtype == TAMD_BF16) return dispatch_mm_bf16(a, block_m, grid_m, st);
     if (a.x_dtype == TAMD_F16) return dispatch_mm_f16(a, block_m, grid_m, st);
@@ -66,8 +68,8 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
       block_m = a.block_m;
       grid_m = a.grid_m;
     } else {
-      block_m = a.force_variant ? a.force_variant : (a.M <= 16 ? 16 : a.M <= 32 ? 32 : a.M <= 64 ? 64 : 128);
-      grid_m = ((a.M + block_m - 1) / block_m) * a.n_experts;
+      block_m = a.force_variant;
+      grid_m = block_m ? ((a.M + block_m - 1) / block_m) * a.n_experts : 0;
     }
     if (a.x_dtype == TAMD_BF16) return dispatch_mm_w16_bf16(a, block_m, grid_m, st);
     return dispatch_mm_w16_f16(a, block_m, grid_m, st);

@@ -182,6 +182,7 @@ int launch_w16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
 // the kernel does not cover.
 template <int XDT>
 int dispatch_w16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  dense_grid(a, block_m, grid_m);
   const bool kc = a.w_stride_k == 1, nc = a.w_stride_n == 1;
   if (!kc && !nc) return TAMD_E_UNSUPPORTED;
   if (a.K % 8 != 0) return TAMD_E_UNSUPPORTED;  // whole 16-byte chunks along K

@@ -6,6 +6,11 @@
 
 namespace tamd {
 int dispatch_mm_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  if (block_m == 0 && a.M <= 256 && stream16_applicable(a)) {
+    // dense with few rows: row blocks of 16 through the streaming kernel (every CU busy, weights re-read from L2)
+    block_m = 16;
+    grid_m = ((a.M + 15) / 16) * a.n_experts;
+  }
   if (block_m == 16 && stream16_applicable(a)) {
     if (a.activation == TAMD_ACT_SWIGLU) return launch_stream16<TAMD_F16, TAMD_ACT_SWIGLU>(a, grid_m, st);
     return launch_stream16<TAMD_F16, TAMD_ACT_NONE>(a, grid_m, st);
