@@ -35,6 +35,8 @@ WORKLOADS = {
     "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
     # down projection + combine: fp8 (per-tensor scaled) expert-sorted rows x MXFP4 W2, gate weights, scatter, k-way sum
     "fc2_combine": dict(T=16384, E=32, k=4, K=2880, N=2880, act=False, fc2=True),
+    # BASELINE config 1: one dense bf16 x MXFP4 product with bias (launch / latency bound: 7.6 MB, 4.3 GFLOP)
+    "c1_dense": dict(M=256, K=2048, N=4096, dense=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
     # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
     "hbm_copy": dict(bytes=1 << 30),
@@ -66,6 +68,57 @@ def hbm_copy(args):
                       "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel_ms": round(ms, 4)},
                       "cpu_baseline": None}))
+
+
+def run_dense(args, cfg):
+    """BASELINE config 1: y = x . deq(W) + bias, x bf16 [M, K], W MXFP4 [K, N] quantised along K."""
+    from oracle import matmul_ref as MR
+    from triton_amd.matmul import PrecisionConfig, matmul
+    M, K, N = cfg["M"], cfg["K"], cfg["N"]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    x_cpu = torch.randn(M, K).to(torch.bfloat16)
+    bias_cpu = (torch.randn(N) * 0.01).to(torch.bfloat16)
+    vals, scales = make_weights(1, K, N, dev)
+    vals, scales = vals[0], scales[0]
+    x, bias = x_cpu.to(dev), bias_cpu.to(dev)
+    pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
+    for _ in range(args.warmup):
+        y = matmul(x, vals, bias, precision_config=pc)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in events:
+        a.record()
+        y = matmul(x, vals, bias, precision_config=pc)
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    flops = 2.0 * M * K * N
+    alg_bytes = M * K * 2 + K // 2 * N + K // 32 * N + N * 2 + M * N * 2
+    torch.set_num_threads(os.cpu_count())
+    t0 = time.perf_counter()
+    ref = MR.matmul_ref(x_cpu, vals.cpu(), bias_cpu, b_mx_scale=scales.cpu())
+    cpu_s = time.perf_counter() - t0
+    ok = bool(torch.allclose(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2))
+    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "moe_matmul_ogs_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x mxfp4 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: dense matmul + bias, M={M}, K={K}, N={N}, W mxfp4 [{K},{N}]",
+                   "scale_layout": args.scale_layout},
+        "matmul_kernel_tflops": round(flops / (kernel_ms * 1e-3) / 1e12, 2),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_stream16_kernel",
+                     "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes, "algorithmic_flops": flops,
+                     "note": "event pairs around one launch include launch latency; the problem is latency bound"},
+        "cpu_baseline": {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                         "sample": f"oracle matmul_ref on the whole problem, {cpu_s:.2f} s"},
+        "parity": {"gemm_within_1e-2": ok}}))
 
 
 def make_weights(E, K, N, device, seed=0):
@@ -244,6 +297,10 @@ def main():
 
     if args.workload == "hbm_copy":
         hbm_copy(args)
+        return
+
+    if WORKLOADS[args.workload].get("dense"):
+        run_dense(args, WORKLOADS[args.workload])
         return
 
     if WORKLOADS[args.workload].get("fc2"):
