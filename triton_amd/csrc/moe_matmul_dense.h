@@ -142,7 +142,7 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
     compute(it);
   }
   wait_dma();
-  tile_epilogue<NFR, ACT>(a, t, acc, lds);
+  tile_epilogue<NFR, ACT, XDT>(a, t, acc, lds);
 }
 
 template <int XDT, int BM, int ACT, bool WKC>

@@ -177,6 +177,13 @@ TAMD_DEVICE void dma16(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t so
                : "memory", "m0");
 }
 TAMD_DEVICE void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding).
+template <int N>
+TAMD_DEVICE void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+  asm volatile("" ::: "memory");
+}
 
 TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
   uint64_t p = (uint64_t)base;
@@ -189,19 +196,24 @@ constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K
 
 // Epilogue of one output tile (shared by every tiled kernel).  The accumulators hold, for fragment
 // (i, f), element j: row 32i + 8(j/4) + 4h + j%4, column t.n0 + wave*64 + c32*NF + f.
-template <int NFR, int ACT>
-TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
+//
+// YDT: output type fixed at compile time, or -1 to read a.y_dtype; ROWSC: per-row betas / gammas may be
+// present; FLEX: flexpoint output (expected / actual scale) may be present.  Everything that is false or
+// fixed here is a branch less per output element, and a tile has up to 160 x 256 of them.
+template <int NFR, int ACT, int YDT, bool ROWSC, bool FLEX>
+TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
   const int c32 = lane % 32, h = lane / 32;
   const int N = a.N;
   const int col0 = t.n0 + wave * 64 + c32 * NF;
-  // ---- epilogue.  Accumulator element j of fragment (i, f): row 32i + 8(j/4) + 4h + j%4,
-  // column col0 + f.  16-bit outputs are staged through LDS (the K stages are dead by now) so
-  // that the global stores are 16 bytes per lane and whole rows of the tile are contiguous.
+  const int ydt = YDT < 0 ? a.y_dtype : YDT;
+  // 16-bit and 8-bit outputs are staged through LDS (the K stages are dead by now) so that the global
+  // stores are 16 bytes per lane and whole rows of the tile are contiguous.
   float flex = 1.0f;
   if (a.x_scale) flex *= *a.x_scale;
   if (a.w_scale) flex *= *a.w_scale;
+  flex *= a.out_alpha;
   float bias[NF];
 #pragma unroll
   for (int f = 0; f < NF; ++f)
@@ -213,17 +225,21 @@ TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_
   const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
   const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
   const bool has_limit = a.act_has_limit != 0;
-  const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
+  const int osz = ydt == TAMD_F32 ? 4 : (ydt == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
   const bool staged = osz < 4;
   // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
-  const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
-  const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
-  const float out_max = max_finite_of(a.y_dtype);
+  const float inv_expected = (FLEX && a.y_expected_scale) ? 1.0f / *a.y_expected_scale : 1.0f;
+  const bool clamp_out = FLEX && a.y_expected_scale != nullptr && a.y_saturate_inf != 0;
+  const float out_max = max_finite_of(ydt);
+  const bool track_max = FLEX && a.y_actual_scale != nullptr;
   uint32_t amax = 0;
   auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
-    return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v)
-                                  : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
+    return ydt == TAMD_BF16 ? f32_to_bf16_bits(v) : (ydt == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
   };
+  // without per-row factors bias * beta * out_alpha is one value per column
+  float bias_a[NF];
+#pragma unroll
+  for (int f = 0; f < NF; ++f) bias_a[f] = bias[f] * a.out_alpha;
   uint8_t *ob = lds;  // [rows][OUT_COLS] outputs of osz bytes
   __syncthreads();
 #pragma unroll
@@ -231,28 +247,40 @@ TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
       const int r = i * 32 + (j >> 2) * 8 + h * 4 + (j & 3);
-      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
-      const float beta = a.betas ? a.betas[erow] : 1.0f;
-      const float gamma = a.gammas ? a.gammas[erow] : 1.0f;
       float v[NF];
+      float gamma = 1.0f;
+      if constexpr (ROWSC) {
+        const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
+        const float beta = a.betas ? a.betas[erow] : 1.0f;
+        gamma = a.gammas ? a.gammas[erow] : 1.0f;
 #pragma unroll
-      for (int f = 0; f < NF; ++f) v[f] = (acc[i][f][j] * flex + bias[f] * beta) * a.out_alpha;
-      float o[NO];
-      if constexpr (ACT == TAMD_ACT_SWIGLU) {
-        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit) * gamma;
+        for (int f = 0; f < NF; ++f) v[f] = __builtin_fmaf(acc[i][f][j], flex, bias_a[f] * beta);
       } else {
 #pragma unroll
-        for (int p = 0; p < NO; ++p) o[p] = v[p] * gamma;
+        for (int f = 0; f < NF; ++f) v[f] = __builtin_fmaf(acc[i][f][j], flex, bias_a[f]);
       }
-      if (a.y_actual_scale && r < t.rows) {
+      float o[NO];
+      if constexpr (ACT == TAMD_ACT_SWIGLU) {
+        o[0] = swiglu_fast(v[0], v[1], a.act_alpha, a.act_limit, has_limit);
+      } else {
 #pragma unroll
-        for (int p = 0; p < NO; ++p)
-          if (out_col0 + p < n_out) amax = absmax_bits(amax, o[p]);
+        for (int p = 0; p < NO; ++p) o[p] = v[p];
       }
+      if constexpr (ROWSC) {
 #pragma unroll
-      for (int p = 0; p < NO; ++p) {
-        o[p] *= inv_expected;
-        if (clamp_out) o[p] = __builtin_fminf(__builtin_fmaxf(o[p], -out_max), out_max);
+        for (int p = 0; p < NO; ++p) o[p] *= gamma;
+      }
+      if constexpr (FLEX) {
+        if (track_max && r < t.rows) {
+#pragma unroll
+          for (int p = 0; p < NO; ++p)
+            if (out_col0 + p < n_out) amax = absmax_bits(amax, o[p]);
+        }
+#pragma unroll
+        for (int p = 0; p < NO; ++p) {
+          o[p] *= inv_expected;
+          if (clamp_out) o[p] = __builtin_fminf(__builtin_fmaxf(o[p], -out_max), out_max);
+        }
       }
       if (staged) {
         uint8_t *dstl = ob + (r * OUT_COLS + wave * 32 * NO + c32 * NO) * osz;
@@ -275,17 +303,19 @@ TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_
       }
     }
   }
-  if (a.y_actual_scale) {
-    // wave maximum, then one atomic per wave; positive floats order like their bit patterns
+  if constexpr (FLEX) {
+    if (track_max) {
+      // wave maximum, then one atomic per wave; positive floats order like their bit patterns
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
-      amax = other > amax ? other : amax;
-    }
-    if (lane == 0) {
-      amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
-      const float sc = __builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f);
-      atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(sc));
+      for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)amax, o);
+        amax = other > amax ? other : amax;
+      }
+      if (lane == 0) {
+        amax = amax < 0x7F800000u ? amax : 0x7F800000u;  // NaN counts as +inf
+        const float sc = __builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f);
+        atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(sc));
+      }
     }
   }
   if (staged) {
@@ -309,6 +339,19 @@ TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_
         for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
       }
     }
+  }
+}
+
+// FAST_YDT: the 16-bit output type that gets the specialised epilogues (the activations' type; bf16 for fp8
+// activations); any other combination takes the general one.
+template <int NFR, int ACT, int FAST_YDT>
+TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
+  const bool flexo = a.y_expected_scale != nullptr || a.y_actual_scale != nullptr;
+  if (a.y_dtype == FAST_YDT && !flexo) {
+    if (a.betas || a.gammas) tile_epilogue_t<NFR, ACT, FAST_YDT, true, false>(a, t, acc, lds);
+    else tile_epilogue_t<NFR, ACT, FAST_YDT, false, false>(a, t, acc, lds);
+  } else {
+    tile_epilogue_t<NFR, ACT, -1, true, true>(a, t, acc, lds);
   }
 }
 
@@ -546,7 +589,9 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       issue_b((it >> 1) + 1);
       compute(it, std::integral_constant<int, 0>{});
       if (it + 1 < n_ka) {
-        wait_dma();
+        // the weight copies just issued (4, after the activation stage it + 1) are not needed before the next
+        // even stage and take the longest (weights stream from HBM, activations mostly hit L2): leave them in flight
+        wait_vmcnt<4>();
         __syncthreads();
         issue_a(it + 2);
         compute(it + 1, std::integral_constant<int, 1>{});
@@ -555,7 +600,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   wait_dma();
 
-  tile_epilogue<NFR, ACT>(a, t, acc, lds);
+  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT>(a, t, acc, lds);
 }
 
 // Row fragments a workgroup can hold: a 128-row block of 16-bit activations also takes a remainder of

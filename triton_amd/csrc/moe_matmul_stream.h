@@ -62,14 +62,6 @@ TAMD_DEVICE void dma4(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t sof
                : "memory", "m0");
 }
 
-// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding).
-template <int N>
-TAMD_DEVICE void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
-  asm volatile("" ::: "memory");
-}
-
 // 16-byte copies with an instruction offset: OFF is added to the global offset and to the LDS address
 // alike, so one M0 value serves up to four consecutive 1 KB pieces of a linear image.
 // SETM0: also loads M0 with lds_addr first (with the wait states an SGPR operand written by a
