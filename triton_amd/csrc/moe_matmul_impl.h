@@ -241,6 +241,18 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
 #pragma unroll
   for (int f = 0; f < NF; ++f) bias_a[f] = bias[f] * a.out_alpha;
   uint8_t *ob = lds;  // [rows][OUT_COLS] outputs of osz bytes
+  // per-row factors: lane L fetches those of row L % 32 of every fragment up front (one round trip to memory);
+  // an element then takes its row's pair from that lane
+  float beta_of[NFR], gamma_of[NFR];
+  if constexpr (ROWSC) {
+#pragma unroll
+    for (int i = 0; i < NFR; ++i) {
+      const int r = i * 32 + c32;
+      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
+      beta_of[i] = a.betas ? a.betas[erow] : 1.0f;
+      gamma_of[i] = a.gammas ? a.gammas[erow] : 1.0f;
+    }
+  }
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < NFR; ++i) {
@@ -250,9 +262,9 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
       float v[NF];
       float gamma = 1.0f;
       if constexpr (ROWSC) {
-        const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
-        const float beta = a.betas ? a.betas[erow] : 1.0f;
-        gamma = a.gammas ? a.gammas[erow] : 1.0f;
+        const int src_lane = (j >> 2) * 8 + h * 4 + (j & 3);
+        const float beta = __shfl(beta_of[i], src_lane);
+        gamma = __shfl(gamma_of[i], src_lane);
 #pragma unroll
         for (int f = 0; f < NF; ++f) v[f] = __builtin_fmaf(acc[i][f][j], flex, bias_a[f] * beta);
       } else {
@@ -323,20 +335,33 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
     const int epc = 16 / osz;                 // outputs per 16-byte chunk
     const int cpr = OUT_COLS / epc;           // chunks per tile row
     const int n_chunks = t.rows * cpr;
-    for (int id = tid; id < n_chunks; id += 256) {
-      const int r = id / cpr, c = (id - r * cpr) * epc;
-      int64_t dst = t.start_m + t.off_m + r;
-      if (a.scatter_indx) dst = a.scatter_indx[dst];
-      if (dst < 0) continue;
-      const int gcol = tile_out0 + c;
-      if (gcol >= n_out) continue;
-      uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * osz;
-      const uint8_t *sp = ob + (r * OUT_COLS + c) * osz;
-      if (gcol + epc <= n_out && ((uintptr_t)yp & 15) == 0) {
-        *(uint4 *)yp = *(const uint4 *)sp;
-      } else {
-        const int n_b = (n_out - gcol < epc ? n_out - gcol : epc) * osz;
-        for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
+    // eight chunks per thread at a time, so that the scatter indices of a batch are fetched together
+    for (int id0 = tid; id0 < n_chunks; id0 += 256 * 8) {
+      int64_t dsts[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int id = id0 + u * 256;
+        const int r = id / cpr;
+        dsts[u] = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);
+        if (a.scatter_indx) dsts[u] = a.scatter_indx[dsts[u]];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int id = id0 + u * 256;
+        if (id >= n_chunks) break;
+        const int r = id / cpr, c = (id - r * cpr) * epc;
+        const int64_t dst = dsts[u];
+        if (dst < 0) continue;
+        const int gcol = tile_out0 + c;
+        if (gcol >= n_out) continue;
+        uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * osz;
+        const uint8_t *sp = ob + (r * OUT_COLS + c) * osz;
+        if (gcol + epc <= n_out && ((uintptr_t)yp & 15) == 0) {
+          *(uint4 *)yp = *(const uint4 *)sp;
+        } else {
+          const int n_b = (n_out - gcol < epc ? n_out - gcol : epc) * osz;
+          for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
+        }
       }
     }
   }
