@@ -44,7 +44,34 @@ __global__ __launch_bounds__(256) void reduce_kernel(const void *__restrict__ x,
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
-    for (int64_t r = 0; r < R; ++r) {
+    int64_t r = 0;
+    if constexpr (VEC == 8) {
+      // plain sums (no mask, no scale: the top-k combine) fetch four rows at a time so that their loads overlap;
+      // the additions keep the order r = 0, 1, 2, ...
+      if (!scale && !mask) {
+        const uint16_t *xp = (const uint16_t *)x + s0 * xs0 + c0;
+        for (; r + 4 <= R; r += 4) {
+          uint4 q[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) q[u] = *(const uint4 *)(xp + (r + u) * xsr);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const uint32_t w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              if constexpr (XDT == TAMD_BF16) {
+                acc[2 * j] += bf16_bits_to_f32(w[j] & 0xFFFFu);
+                acc[2 * j + 1] += bf16_bits_to_f32(w[j] >> 16);
+              } else {
+                acc[2 * j] += f16_bits_to_f32(w[j] & 0xFFFFu);
+                acc[2 * j + 1] += f16_bits_to_f32(w[j] >> 16);
+              }
+            }
+          }
+        }
+      }
+    }
+    for (; r < R; ++r) {
       float v[VEC];
       if constexpr (VEC == 1) {
         v[0] = load_as_f32<XDT>(x, s0 * xs0 + r * xsr + c0 * xs1);
