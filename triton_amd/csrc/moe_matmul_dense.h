@@ -10,7 +10,7 @@
 //     its column with 2-byte LDS reads.  The MFMA wants K-contiguous operands on both sides, so one of
 //     the two has to be transposed somewhere; doing it on the LDS read costs no extra pass.
 //
-// One workgroup per CU (the two 32 KB weight stages need the LDS); not a tuned kernel -- the unquantised
+// One workgroup per CU (three 32 KB weight stages); not a tuned kernel -- the unquantised
 // products on this path are small next to the expert matmuls.
 #pragma once
 #include "moe_matmul_impl.h"
@@ -37,7 +37,8 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
   const int64_t w_span = (WKC ? (int64_t)N * a.w_stride_n : (int64_t)K * a.w_stride_k) * 2;
   const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e * 2, (uint32_t)w_span);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-  const uint32_t lds_b = lds_base + 2 * A_STAGE;
+  constexpr int RING = 3;  // stages: one consumed, two in flight (the K loop of a small tile is latency bound)
+  const uint32_t lds_b = lds_base + RING * A_STAGE;
 
   // ---- activation DMA (as in run_tile): lane -> (row 8w + lane/8, slot lane%8)
   const int a_rin = wave * 8 + lane / 8;
@@ -81,14 +82,14 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
       for (int j = 0; j < 16; ++j) acc[i][f][j] = 0.f;
 
   const int n_k = (K + KA - 1) / KA;
-  auto issue = [&](int it) {  // clamped: past the end the last stage is copied again (never read)
+  auto issue = [&](int it, int slot) {  // clamped: past the end the last stage is copied again (never read)
     it = it < n_k ? it : n_k - 1;
     const int kb = it * KA;
     const uint32_t akill = kb + a_chunk * 8 < K ? 0u : kOob;
-    const uint32_t sa = lds_base + (it & 1) * A_STAGE + wave * 8 * A_ROW_BYTES;
+    const uint32_t sa = lds_base + slot * A_STAGE + wave * 8 * A_ROW_BYTES;
 #pragma unroll
     for (int i = 0; i < NFR; ++i) dma16(rx, sa + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * 2);
-    const uint32_t sb = lds_b + (it & 1) * W16_STAGE;
+    const uint32_t sb = lds_b + slot * W16_STAGE;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if constexpr (WKC) {
@@ -103,9 +104,9 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
     }
   };
 
-  auto compute = [&](int it) {
-    const uint8_t *abuf = lds + (it & 1) * A_STAGE;
-    const uint8_t *bbuf = lds + 2 * A_STAGE + (it & 1) * W16_STAGE;
+  auto compute = [&](int slot) {
+    const uint8_t *abuf = lds + slot * A_STAGE;
+    const uint8_t *bbuf = lds + RING * A_STAGE + slot * W16_STAGE;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       frag_t af[NFR];
@@ -134,12 +135,15 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
     }
   };
 
-  issue(0);
+  issue(0, 0);
+  issue(1, 1);
+  int rd = 0;  // ring slot of the stage being consumed (stage it lives in slot it % 3)
   for (int it = 0; it < n_k; ++it) {
-    wait_dma();
-    __syncthreads();  // stage `it` is visible; everyone is done with the buffer stage it + 1 goes to
-    issue(it + 1);
-    compute(it);
+    wait_vmcnt<NFR + 8>();  // copies complete in order: all but the NFR + 8 of stage it + 1 have landed
+    __syncthreads();        // stage `it` is visible; everyone is done with the slot stage it + 2 goes to
+    issue(it + 2, rd == 0 ? 2 : rd - 1);
+    compute(rd);
+    rd = rd == 2 ? 0 : rd + 1;
   }
   wait_dma();
   tile_epilogue<NFR, ACT, XDT>(a, t, acc, lds);
@@ -164,7 +168,8 @@ template <int XDT, int BM, int ACT, bool WKC>
 int launch_w16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int MF = BM <= 32 ? 1 : BM / 32;
   constexpr int LDS_ROWS = 32 * MF;
-  constexpr int PIPE = 2 * LDS_ROWS * A_ROW_BYTES + 2 * W16_STAGE;
+  constexpr int PIPE = 3 * LDS_ROWS * A_ROW_BYTES + 3 * W16_STAGE;
+  static_assert(PIPE <= 160 * 1024, "one workgroup per CU");
   constexpr int OUT_BYTES = LDS_ROWS * 256 * 2;
   const int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
   const int64_t total = (int64_t)grid_m * grid_n;
