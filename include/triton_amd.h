@@ -61,6 +61,8 @@ const char *tamd_error_string(int code);
  * out_vals gets L/2 bytes (mxfp4) contiguous along the quantised axis for every
  * (b, r): byte j of run (b, r) holds codes 2j (low nibble) and 2j+1.
  * out_scales gets L/32 e8m0 bytes per (b, r), contiguous likewise.
+ * out_dtype TAMD_FP8_E4M3 / TAMD_FP8_E5M2 (MXFP8: one byte per element, clamped to the finite range and rounded to
+ * nearest even, mxfp.py:313-316) is built for src_stride_l == 1 only; other layouts return TAMD_E_UNSUPPORTED.
  */
 int tamd_downcast_mxfp(const void *src, int src_dtype, int64_t nb, int64_t L, int64_t nr,
                        int64_t src_stride_b, int64_t src_stride_l, int64_t src_stride_r,
@@ -76,7 +78,8 @@ int tamd_downcast_mxfp(const void *src, int src_dtype, int64_t nb, int64_t L, in
  * along the quantised axis, strides for b and r given).  dst is [nb, L, nr] with
  * either dst_stride_l == 1 or dst_stride_r == 1.  A scale byte of 0xFF yields
  * NaN, 0x00 multiplies by +0.0; results are clamped to the finite range of
- * dst_dtype (F32 / F16 / BF16).
+ * dst_dtype (F32 / F16 / BF16).  val_dtype TAMD_FP8_E4M3 / TAMD_FP8_E5M2 (one byte per element; e5m2
+ * infinities pass through, mxfp.py:438-440) needs dst_stride_l == 1.
  */
 int tamd_upcast_mxfp(const void *vals, int val_dtype, int64_t val_stride_b, int64_t val_stride_r,
                      const uint8_t *scales, int64_t scale_stride_b, int64_t scale_stride_r,

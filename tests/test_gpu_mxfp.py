@@ -106,3 +106,55 @@ def test_pitched_input(device):
     rv, rs = downcast_to_mxfp_ref(x, torch.uint8, 1)
     v, s = downcast_to_mxfp(big.to(device)[:, :256], torch.uint8, axis=1)
     assert torch.equal(v.cpu(), rv) and torch.equal(s.cpu(), rs)
+
+
+# ---------------------------------------------------------------------------- fp8 values (MXFP8)
+
+FP8_TYPES = [torch.float8_e4m3fn, torch.float8_e5m2]
+
+
+@pytest.mark.parametrize("shape,axis", [((256, 2880), 1), ((3, 96, 224), -1), ((7, 32), 1), ((2048, 96), 0), ((4, 64, 6), 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("vdt", FP8_TYPES)
+@pytest.mark.parametrize("mode", list(DequantScaleRoundingMode))
+def test_mxfp8_downcast_matches_oracle(shape, axis, dtype, vdt, mode, device):
+    torch.manual_seed(0)
+    x = (torch.randn(shape) * torch.exp(torch.randn(shape) * 2)).to(dtype)
+    x.view(-1)[::17] = 0
+    ref_v, ref_s = downcast_to_mxfp_ref(x, vdt, axis, "up" if mode.value == 0 else "down")
+    v, s = downcast_to_mxfp(x.to(device), vdt, axis, DEQUANT_SCALE_ROUNDING_MODE=mode)
+    assert v.dtype == vdt and tuple(v.shape) == tuple(x.shape)
+    assert torch.equal(s.cpu(), ref_s), "scales differ"
+    assert torch.equal(v.cpu().view(torch.uint8), ref_v.contiguous().view(torch.uint8)), "values differ"
+
+
+@pytest.mark.parametrize("shape,axis", [((128, 512), 1), ((4, 64, 96), 2), ((96, 40), 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("vdt", FP8_TYPES)
+def test_mxfp8_upcast_matches_oracle(shape, axis, dtype, vdt, device):
+    """Every fp8 byte (NaN codes included) against every scale byte (0 and 0xFF included)."""
+    torch.manual_seed(2)
+    v = torch.randint(0, 256, shape, dtype=torch.uint8).view(vdt)
+    s_shape = list(shape)
+    s_shape[axis] //= 32
+    s = torch.randint(0, 256, s_shape, dtype=torch.uint8)
+    s.view(-1)[:2] = torch.tensor([0, 255], dtype=torch.uint8)
+    out = upcast_from_mxfp(v.to(device), s.to(device), dtype, axis)
+    ref = upcast_from_mxfp_ref(v, s, dtype, axis)
+    a, b = out.cpu().float(), ref.float()
+    assert torch.equal(torch.isnan(a), torch.isnan(b))
+    assert torch.equal(torch.nan_to_num(a), torch.nan_to_num(b))
+
+
+@pytest.mark.parametrize("vdt,max_q", [(torch.float8_e4m3fn, 448.0), (torch.float8_e5m2, 57344.0)])
+@pytest.mark.parametrize("dst", [torch.float32, torch.bfloat16, torch.float16])
+def test_mxfp8_quant_dequant_exact(vdt, max_q, dst, device):
+    """The reference's tests/test_mxfp.py:171-205 for the fp8 value types, quantised along a strided axis."""
+    top = 128.0 if (vdt == torch.float8_e5m2 and dst == torch.float16) else max_q
+    pos = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, top], dtype=dst)
+    k = torch.cat([pos, -pos]).reshape(-1, 1)
+    w = (k * (2.0**torch.arange(-8, 8, dtype=dst)).reshape(1, -1)).repeat(9, 32)
+    w = w.reshape(1, *w.shape).mT.contiguous().mT
+    w = torch.nn.functional.pad(w, (0, 0, 0, 16)).to(device)
+    q, s = downcast_to_mxfp(w, vdt, axis=1)
+    assert torch.equal(upcast_from_mxfp(q, s, dst, axis=1), w)

@@ -203,3 +203,67 @@ def test_ragged_tail_group():
     assert list(q.shape) == [1, 20] and s.tolist() == [[0, 126]]
     d = MX.upcast_from_mxfp_ref(q, s, torch.float32, axis=1)
     assert d[0, 35].item() == 3.0
+
+
+# ---------------------------------------------------------------------------- fp8 values (MXFP8)
+
+FP8_KINDS = [(torch.float8_e4m3fn, 448.0), (torch.float8_e5m2, 57344.0)]
+
+
+@pytest.mark.parametrize("vdt,max_q", FP8_KINDS)
+@pytest.mark.parametrize("dst", [torch.float32, torch.bfloat16, torch.float16])
+def test_fp8_representable_values_roundtrip(vdt, max_q, dst):
+    """tests/test_mxfp.py:171-205 of the reference for the fp8 value types: {0, .5, 1, 1.5, 2, 3, 4, max} x 2^[-8, 8)
+    survive quantise -> dequantise exactly (fp16 cannot hold the e5m2 range: max 128 there, as in the reference)."""
+    top = 128.0 if (vdt == torch.float8_e5m2 and dst == torch.float16) else max_q
+    pos = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, top], dtype=dst)
+    k = torch.cat([pos, -pos]).reshape(-1, 1)
+    w = (k * (2.0**torch.arange(-8, 8, dtype=dst)).reshape(1, -1)).repeat(9, 32)
+    w = torch.nn.functional.pad(w.reshape(1, *w.shape), (0, 0, 0, 16))
+    v, s = MX.downcast_to_mxfp_ref(w, vdt, axis=1)
+    assert v.dtype == vdt and s.dtype == torch.uint8 and tuple(s.shape) == (1, w.shape[1] // 32, w.shape[2])
+    assert torch.equal(MX.upcast_from_mxfp_ref(v, s, dst, axis=1), w)
+
+
+@pytest.mark.parametrize("vdt,max_q", FP8_KINDS)
+@pytest.mark.parametrize("dst,big", [(torch.float16, 65470.0), (torch.bfloat16, 3.3895e38), (torch.float32, 3.3895e38)])
+def test_fp8_extreme_values_stay_finite(vdt, max_q, dst, big):
+    """tests/test_mxfp.py:154-168."""
+    x = torch.tensor([big, big] + [0.0] * 30, dtype=dst)
+    v, s = MX.downcast_to_mxfp_ref(x, vdt, axis=-1)
+    out = MX.upcast_from_mxfp_ref(v, s, dst, axis=-1)
+    assert not out.isinf().any() and not out.isnan().any()
+
+
+@pytest.mark.parametrize("vdt,max_q", FP8_KINDS)
+def test_fp8_scale_closed_form_and_nearest_value(vdt, max_q):
+    """ROUND_UP scale = smallest power of two with max / scale <= max_q; every value is the fp8 number nearest to
+    x / scale (ties to the even code), found by brute force over all 256 codes decoded by torch."""
+    torch.manual_seed(0)
+    x = torch.randn(64, 32) * torch.exp(torch.randn(64, 1) * 3)
+    v, s = MX.downcast_to_mxfp_ref(x, vdt, axis=1)
+    table = torch.arange(256, dtype=torch.uint8).view(vdt).float()
+    finite = torch.isfinite(table)
+    for r in range(64):
+        m = float(x[r].abs().max())
+        e = int(s[r, 0]) - 127
+        assert m / 2.0**e <= max_q and (m / 2.0**(e - 1) > max_q)
+        q = (x[r].double() / 2.0**e)
+        d = (table[finite].double()[None, :] - q[:, None]).abs()
+        best = d.min(dim=1).values
+        got = v[r].float().double()
+        assert torch.all((got - q).abs() <= best + 1e-300)
+        # ties: the chosen code has an even mantissa bit pattern
+        tie = (d <= best[:, None]).sum(dim=1) > 1
+        if tie.any():
+            assert torch.all((v[r].view(torch.uint8)[tie] & 1) == 0)
+
+
+def test_fp8_round_down_uses_largest_power_of_two():
+    """mxfp_details/_downcast_to_mxfp.py:24-31: ROUND_DOWN divides by 256 (e4m3) / 32768 (e5m2) and truncates."""
+    x = torch.zeros(1, 32)
+    x[0, 0] = 300.0
+    for vdt, p2 in ((torch.float8_e4m3fn, 256.0), (torch.float8_e5m2, 32768.0)):
+        _, s = MX.downcast_to_mxfp_ref(x, vdt, axis=1, rounding="down")
+        import math
+        assert int(s[0, 0]) == 127 + math.floor(math.log2(300.0 / p2))

@@ -1,4 +1,4 @@
-// MXFP4 quantise / dequantise for gfx950.  Bandwidth kernels: 128-bit global
+// MXFP4 / MXFP8 quantise / dequantise for gfx950.  Bandwidth kernels: 128-bit global
 // accesses, one 32-element group handled by 4 lanes (quantised axis contiguous)
 // or by one lane per column (quantised axis strided, i.e. the weight layout).
 //
@@ -19,13 +19,22 @@ TAMD_DEVICE uint32_t e2m1_code(float q) {
   return c | ((f32_to_bits(q) >> 28) & 8u);
 }
 
+// Value kinds of a microscaled tensor: e2m1 codes (two per byte), or fp8 bytes.  Largest magnitude and
+// largest power of two of each (mxfp.py:206-209, mxfp_details/_downcast_to_mxfp.py:24-31).
+constexpr int QK_E2M1 = 0, QK_E4M3 = 1, QK_E5M2 = 2;
+template <int QK>
+constexpr float kMaxQ = QK == QK_E2M1 ? 6.0f : (QK == QK_E4M3 ? 448.0f : 57344.0f);
+template <int QK>
+constexpr float kInvPow2Q = QK == QK_E2M1 ? 0.25f : (QK == QK_E4M3 ? 1.0f / 256.0f : 1.0f / 32768.0f);
+
 // Returns the multiplier 1/scale and writes the e8m0 byte.
+template <int QK = QK_E2M1>
 TAMD_DEVICE float group_scale(float gmax, int mode, uint32_t &scale_byte) {
   uint32_t sb;
   if (mode == TAMD_ROUND_UP) {
-    sb = (f32_to_bits(gmax / 6.0f) + 0x007FFFFFu) & 0x7F800000u;
+    sb = (f32_to_bits(gmax / kMaxQ<QK>) + 0x007FFFFFu) & 0x7F800000u;
   } else {
-    sb = f32_to_bits(gmax * 0.25f) & 0x7F800000u;
+    sb = f32_to_bits(gmax * kInvPow2Q<QK>) & 0x7F800000u;
   }
   scale_byte = sb >> 23;
   float ds = bits_to_f32(sb);
@@ -38,15 +47,31 @@ TAMD_DEVICE float e2m1_value(uint32_t code) {
   return bits_to_f32(bits | ((code & 8u) << 28));
 }
 
+// q (already multiplied by 1/scale) -> fp8 byte: clamp to the finite range, round to nearest even (mxfp.py:313-316)
+template <int QK>
+TAMD_DEVICE uint32_t fp8_code(float q) {
+  if (q != q) return 0x7Fu;
+  const float c = __builtin_fminf(__builtin_fmaxf(q, -kMaxQ<QK>), kMaxQ<QK>);
+  if constexpr (QK == QK_E4M3) return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xFFu;
+  return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(c, c, 0, false) & 0xFFu;
+}
+template <int QK>
+TAMD_DEVICE float fp8_value(uint32_t byte) {
+  if constexpr (QK == QK_E4M3) return __builtin_amdgcn_cvt_f32_fp8((int)byte, 0);
+  return __builtin_amdgcn_cvt_f32_bf8((int)byte, 0);
+}
+
 template <int DT>
 constexpr float kMaxFinite =
     DT == TAMD_F32 ? 3.4028234663852886e+38f : (DT == TAMD_BF16 ? 3.3895313892515355e+38f : 65504.f);
 
-template <int DT>
+template <int DT, int QK = QK_E2M1>
 TAMD_DEVICE float dequant_one(uint32_t code, float mult, bool is_nan) {
-  float v = e2m1_value(code) * mult;
+  float v = (QK == QK_E2M1 ? e2m1_value(code) : fp8_value<QK>(code)) * mult;
   constexpr float mf = kMaxFinite<DT>;
   v = v != v ? v : __builtin_fminf(__builtin_fmaxf(v, -mf), mf);
+  // e5m2 has infinities: they pass through whatever the scale is (mxfp.py:438-440 of the reference)
+  if (QK == QK_E5M2 && (code & 0x7Fu) == 0x7Cu) v = bits_to_f32(0x7F800000u | ((code & 0x80u) << 24));
   return is_nan ? bits_to_f32(0x7FC00000u) : v;
 }
 
@@ -59,7 +84,7 @@ TAMD_DEVICE uint32_t pack2(float a, float b) {
 // ---------------------------------------------------------------------------
 // downcast, quantised axis contiguous in the source: 4 lanes x 8 elements per group
 // ---------------------------------------------------------------------------
-template <int DT, bool VEC>
+template <int DT, bool VEC, int QK>
 __global__ __launch_bounds__(256) void downcast_rows_kernel(
     const void *__restrict__ src, int64_t n_groups_total, int64_t G, int64_t nr, int64_t ssb, int64_t ssr,
     uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
@@ -100,12 +125,23 @@ __global__ __launch_bounds__(256) void downcast_rows_kernel(
   m = __builtin_fmaxf(m, __shfl_xor(m, 1));
   m = __builtin_fmaxf(m, __shfl_xor(m, 2));
   uint32_t sbyte;
-  float qs = group_scale(m, mode, sbyte);
-  uint32_t packed = 0;
+  float qs = group_scale<QK>(m, mode, sbyte);
+  if constexpr (QK == QK_E2M1) {
+    uint32_t packed = 0;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] * qs) << (4 * j);
-  if (!live) return;
-  *(uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4) = packed;
+    for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] * qs) << (4 * j);
+    if (!live) return;
+    *(uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4) = packed;
+  } else {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      lo |= fp8_code<QK>(v[j] * qs) << (8 * j);
+      hi |= fp8_code<QK>(v[4 + j] * qs) << (8 * j);
+    }
+    if (!live) return;
+    *(uint2 *)(vals + b * vsb + r * vsr + g * 32 + sub * 8) = make_uint2(lo, hi);
+  }
   if (sub == 0) scales[b * csb + r * csr + g] = (uint8_t)sbyte;
 }
 
@@ -179,7 +215,7 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
 // ---------------------------------------------------------------------------
 // upcast, destination contiguous along the quantised axis
 // ---------------------------------------------------------------------------
-template <int DT>
+template <int DT, int QK>
 __global__ __launch_bounds__(256) void upcast_rows_kernel(
     const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
     int64_t csb, int64_t csr, void *__restrict__ dst, int64_t n_groups_total, int64_t G, int64_t nr,
@@ -189,13 +225,22 @@ __global__ __launch_bounds__(256) void upcast_rows_kernel(
   if (gid >= n_groups_total) return;
   int64_t run = gid / G, g = gid - run * G;
   int64_t b = run / nr, r = run - b * nr;
-  uint32_t packed = *(const uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4);
   uint32_t s = scales[b * csb + r * csr + g];
   float mult = bits_to_f32(s << 23);
   bool is_nan = s == 0xFFu;
   float o[8];
+  if constexpr (QK == QK_E2M1) {
+    uint32_t packed = *(const uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) o[j] = dequant_one<DT>((packed >> (4 * j)) & 0xFu, mult, is_nan);
+    for (int j = 0; j < 8; ++j) o[j] = dequant_one<DT>((packed >> (4 * j)) & 0xFu, mult, is_nan);
+  } else {
+    const uint2 w = *(const uint2 *)(vals + b * vsb + r * vsr + g * 32 + sub * 8);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[j] = dequant_one<DT, QK>((w.x >> (8 * j)) & 0xFFu, mult, is_nan);
+      o[4 + j] = dequant_one<DT, QK>((w.y >> (8 * j)) & 0xFFu, mult, is_nan);
+    }
+  }
   int64_t off = b * dsb + r * dsr + g * 32 + sub * 8;
   if (vec_ok) {
     if constexpr (DT == TAMD_F32) {
@@ -262,7 +307,7 @@ __global__ __launch_bounds__(256) void upcast_cols_kernel(
   }
 }
 
-template <int DT>
+template <int DT, int QK>
 int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t ssb, int64_t ssl, int64_t ssr,
                     uint8_t *vals, int64_t vsb, int64_t vsr, uint8_t *scales, int64_t csb, int64_t csr,
                     int mode, hipStream_t st) {
@@ -274,14 +319,15 @@ int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t 
     int64_t blocks = (total + 63) / 64;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
     if (vec)
-      downcast_rows_kernel<DT, true><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
+      downcast_rows_kernel<DT, true, QK><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
                                                                             vsb, vsr, scales, csb, csr, mode);
     else
-      downcast_rows_kernel<DT, false><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
+      downcast_rows_kernel<DT, false, QK><<<dim3((unsigned)blocks), 256, 0, st>>>(src, total, G, nr, ssb, ssr, vals,
                                                                              vsb, vsr, scales, csb, csr, mode);
     return launch_status();
   }
   if (ssr != 1) return TAMD_E_INVALID;
+  if constexpr (QK != QK_E2M1) return TAMD_E_UNSUPPORTED;  // fp8 values: quantised axis contiguous only
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(src, 16) && (ssb * ES) % 16 == 0 && (ssl * ES) % 16 == 0;
   if (vec) {
@@ -298,7 +344,7 @@ int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t 
   return launch_status();
 }
 
-template <int DT>
+template <int DT, int QK>
 int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *scales, int64_t csb, int64_t csr,
                   void *dst, int64_t nb, int64_t L, int64_t nr, int64_t dsb, int64_t dsl, int64_t dsr,
                   hipStream_t st) {
@@ -309,11 +355,12 @@ int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *
     int vec = aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsr * ES) % 16 == 0;
     int64_t blocks = (total + 63) / 64;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-    upcast_rows_kernel<DT><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, total, G,
+    upcast_rows_kernel<DT, QK><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, total, G,
                                                                   nr, dsb, dsr, vec);
     return launch_status();
   }
   if (dsr != 1) return TAMD_E_INVALID;
+  if constexpr (QK != QK_E2M1) return TAMD_E_UNSUPPORTED;  // fp8 values: quantised axis contiguous only
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsl * ES) % 16 == 0;
   if (vec) {
@@ -341,25 +388,27 @@ extern "C" int tamd_downcast_mxfp(const void *src, int src_dtype, int64_t nb, in
                                   int rounding_mode, void *stream) {
   if (nb < 0 || L < 0 || nr < 0 || L % 32 != 0) return TAMD_E_INVALID;
   if (rounding_mode != TAMD_ROUND_UP && rounding_mode != TAMD_ROUND_DOWN) return TAMD_E_INVALID;
-  if (out_dtype != TAMD_MXFP4) return TAMD_E_UNSUPPORTED;
+  if (out_dtype != TAMD_MXFP4 && out_dtype != TAMD_FP8_E4M3 && out_dtype != TAMD_FP8_E5M2) return TAMD_E_INVALID;
   if (nb == 0 || L == 0 || nr == 0) return 0;
   if (!src || !out_vals || !out_scales) return TAMD_E_INVALID;
   if (!aligned(out_vals, 16) || val_stride_b % 16 != 0 || val_stride_r % 16 != 0) return TAMD_E_ALIGNMENT;
   hipStream_t st = (hipStream_t)stream;
   uint8_t *v = (uint8_t *)out_vals;
-  switch (src_dtype) {
-    case TAMD_F32:
-      return launch_downcast<TAMD_F32>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
-                                       val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
-    case TAMD_BF16:
-      return launch_downcast<TAMD_BF16>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
-                                        val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
-    case TAMD_F16:
-      return launch_downcast<TAMD_F16>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,
-                                       val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st);
-    default:
-      return TAMD_E_INVALID;
+#define TAMD_DOWN(DT, QK)                                                                                          \
+  return launch_downcast<DT, QK>(src, nb, L, nr, src_stride_b, src_stride_l, src_stride_r, v, val_stride_b,          \
+                                 val_stride_r, out_scales, scale_stride_b, scale_stride_r, rounding_mode, st)
+#define TAMD_DOWN_SRC(QK)                      \
+  switch (src_dtype) {                         \
+    case TAMD_F32: TAMD_DOWN(TAMD_F32, QK);    \
+    case TAMD_BF16: TAMD_DOWN(TAMD_BF16, QK);  \
+    case TAMD_F16: TAMD_DOWN(TAMD_F16, QK);    \
+    default: return TAMD_E_INVALID;            \
   }
+  if (out_dtype == TAMD_MXFP4) TAMD_DOWN_SRC(QK_E2M1)
+  if (out_dtype == TAMD_FP8_E4M3) TAMD_DOWN_SRC(QK_E4M3)
+  TAMD_DOWN_SRC(QK_E5M2)
+#undef TAMD_DOWN_SRC
+#undef TAMD_DOWN
 }
 
 extern "C" int tamd_upcast_mxfp(const void *vals, int val_dtype, int64_t val_stride_b, int64_t val_stride_r,
@@ -367,23 +416,25 @@ extern "C" int tamd_upcast_mxfp(const void *vals, int val_dtype, int64_t val_str
                                 int dst_dtype, int64_t nb, int64_t L, int64_t nr, int64_t dst_stride_b,
                                 int64_t dst_stride_l, int64_t dst_stride_r, void *stream) {
   if (nb < 0 || L < 0 || nr < 0 || L % 32 != 0) return TAMD_E_INVALID;
-  if (val_dtype != TAMD_MXFP4) return TAMD_E_UNSUPPORTED;
+  if (val_dtype != TAMD_MXFP4 && val_dtype != TAMD_FP8_E4M3 && val_dtype != TAMD_FP8_E5M2) return TAMD_E_INVALID;
   if (nb == 0 || L == 0 || nr == 0) return 0;
   if (!vals || !scales || !dst) return TAMD_E_INVALID;
   if (!aligned(vals, 16) || val_stride_b % 16 != 0 || val_stride_r % 16 != 0) return TAMD_E_ALIGNMENT;
   hipStream_t st = (hipStream_t)stream;
   const uint8_t *v = (const uint8_t *)vals;
-  switch (dst_dtype) {
-    case TAMD_F32:
-      return launch_upcast<TAMD_F32>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
-                                     L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
-    case TAMD_BF16:
-      return launch_upcast<TAMD_BF16>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
-                                      L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
-    case TAMD_F16:
-      return launch_upcast<TAMD_F16>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb,
-                                     L, nr, dst_stride_b, dst_stride_l, dst_stride_r, st);
-    default:
-      return TAMD_E_INVALID;
+#define TAMD_UP(DT, QK)                                                                                              \
+  return launch_upcast<DT, QK>(v, val_stride_b, val_stride_r, scales, scale_stride_b, scale_stride_r, dst, nb, L, nr, \
+                               dst_stride_b, dst_stride_l, dst_stride_r, st)
+#define TAMD_UP_DST(QK)                      \
+  switch (dst_dtype) {                       \
+    case TAMD_F32: TAMD_UP(TAMD_F32, QK);    \
+    case TAMD_BF16: TAMD_UP(TAMD_BF16, QK);  \
+    case TAMD_F16: TAMD_UP(TAMD_F16, QK);    \
+    default: return TAMD_E_INVALID;          \
   }
+  if (val_dtype == TAMD_MXFP4) TAMD_UP_DST(QK_E2M1)
+  if (val_dtype == TAMD_FP8_E4M3) TAMD_UP_DST(QK_E4M3)
+  TAMD_UP_DST(QK_E5M2)
+#undef TAMD_UP_DST
+#undef TAMD_UP
 }

@@ -5,7 +5,7 @@ from enum import Enum
 import torch
 
 from .. import _lib
-from ..tensor import FP4, Tensor, empty, wrap_torch_tensor
+from ..tensor import FP4, Tensor, empty, torch_dtype_to_dtype, wrap_torch_tensor
 from ..tensor_details.dtype import UINT8
 from ..tensor_details.layout import StridedLayout
 
@@ -58,13 +58,20 @@ def downcast_to_mxfp(x, out_dtype, axis: int, scale_dtype: torch.dtype = torch.u
     assert -x.ndim <= axis < x.ndim, f"Invalid axis {axis=}"
     assert out_dtype in (torch.uint8, FP4, torch.float8_e4m3fn, torch.float8_e5m2), f"Invalid output dtype {out_dtype=}"
     assert x.dtype in (torch.float32, torch.bfloat16, torch.float16), f"Invalid input tensor dtype {x.dtype}"
-    if out_dtype not in (torch.uint8, FP4) or scale_dtype != torch.uint8 or microblock_size != MXFP_BLOCK_SIZE:
-        raise NotImplementedError("only e2m1 values with e8m0 scales per 32 elements are built for gfx950")
+    if scale_dtype != torch.uint8 or microblock_size != MXFP_BLOCK_SIZE:
+        raise NotImplementedError("only e8m0 scales per 32 elements are built for gfx950")
     _lib.require_gpu(x, "x")
     axis = axis % x.ndim
     layout = StridedLayout(major_dim=axis - x.ndim)
     L = x.shape[axis]
-    y_value = empty(list(x.shape), FP4, x.device, layout)
+    is_fp4 = out_dtype in (torch.uint8, FP4)
+    value_code = _lib.MXFP4 if is_fp4 else _lib.dtype_code(out_dtype)
+    if not is_fp4 and x.numel() > 0 and x.stride(axis) != 1:
+        # fp8 values are quantised by the kernel for a contiguous axis only: move it last, quantise, move it back
+        vt, st = downcast_to_mxfp(x.transpose(axis, -1).contiguous(), out_dtype, -1, scale_dtype, microblock_size,
+                                  DEQUANT_SCALE_ROUNDING_MODE)
+        return vt.transpose(axis, -1), st.transpose(axis, -1)
+    y_value = empty(list(x.shape), FP4 if is_fp4 else torch_dtype_to_dtype(out_dtype), x.device, layout)
     scale_shape = [*x.shape[:axis], L // microblock_size, *x.shape[axis + 1:]]
     y_scale = empty(scale_shape, UINT8, x.device, layout)
     if x.numel() > 0:
@@ -85,7 +92,7 @@ def downcast_to_mxfp(x, out_dtype, axis: int, scale_dtype: torch.dtype = torch.u
             s.copy_(st.transpose(axis, -1))
             return v, s
         rc = _lib.lib().tamd_downcast_mxfp(_lib.ptr(x), _lib.dtype_code(x.dtype), nb, L, nr, sb, sl, sr,
-                                           _lib.ptr(v), _lib.MXFP4, vv[3], vv[5], _lib.ptr(s), sv[3], sv[5],
+                                           _lib.ptr(v), value_code, vv[3], vv[5], _lib.ptr(s), sv[3], sv[5],
                                            DEQUANT_SCALE_ROUNDING_MODE.value, _lib.stream_ptr(x.device))
         _lib.check(rc, "downcast_to_mxfp")
     return y_value.storage.data, y_scale.storage.data
@@ -102,10 +109,21 @@ def upcast_from_mxfp(tensor: torch.Tensor, scale: torch.Tensor, target_dtype: to
     assert tensor.dtype in {torch.uint8, torch.float8_e5m2, torch.float8_e4m3fn}, f"Invalid tensor dtype {tensor.dtype=}"
     assert scale.dtype == torch.uint8 or scale.dtype == torch.float8_e4m3fn, f"Invalid scale dtype {scale.dtype=}"
     assert target_dtype in (torch.float16, torch.bfloat16, torch.float32), f"Invalid output dtype {target_dtype=}"
-    if tensor.dtype != torch.uint8 or scale.dtype != torch.uint8:
-        raise NotImplementedError("only e2m1 values with e8m0 scales are built for gfx950")
+    if scale.dtype != torch.uint8:
+        raise NotImplementedError("only e8m0 scales are built for gfx950")
     _lib.require_gpu(tensor, "tensor")
-    L = tensor.shape[axis] * 2
+    is_fp4 = tensor.dtype == torch.uint8
+    value_code = _lib.MXFP4 if is_fp4 else _lib.dtype_code(tensor.dtype)
+    L = tensor.shape[axis] * (2 if is_fp4 else 1)
+    if not is_fp4 and axis != ndim - 1:
+        # fp8 values are dequantised by the kernel into a contiguous axis only
+        out = upcast_from_mxfp(tensor.transpose(axis, -1).contiguous(), scale.transpose(axis, -1).contiguous(),
+                               target_dtype, -1, None).transpose(axis, -1).contiguous()
+        if tensor_scale is not None:
+            shape = (1, ) * out.ndim if tensor_scale.numel() == 1 else (*tensor_scale.shape[:axis], 1,
+                                                                        *tensor_scale.shape[axis:])
+            out = out * tensor_scale.to(device=out.device).reshape(shape)
+        return out
     out_shape = [*tensor.shape[:axis], L, *tensor.shape[axis + 1:]]
     out = torch.empty(out_shape, dtype=target_dtype, device=tensor.device)
     if out.numel() > 0:
@@ -118,7 +136,7 @@ def upcast_from_mxfp(tensor: torch.Tensor, scale: torch.Tensor, target_dtype: to
         dsl, dsr = ov[4], ov[5]
         if nr == 1:
             dsl, dsr = 1, 0
-        rc = _lib.lib().tamd_upcast_mxfp(_lib.ptr(tensor), _lib.MXFP4, vv[3], vv[5], _lib.ptr(scale), sv[3], sv[5],
+        rc = _lib.lib().tamd_upcast_mxfp(_lib.ptr(tensor), value_code, vv[3], vv[5], _lib.ptr(scale), sv[3], sv[5],
                                          _lib.ptr(out), _lib.dtype_code(target_dtype), nb, L, nr, ov[3], dsl, dsr,
                                          _lib.stream_ptr(tensor.device))
         _lib.check(rc, "upcast_from_mxfp")
