@@ -219,6 +219,11 @@ typedef struct tamd_matmul_args {
    * tensor_details/layout_details/cdna4_scale.py:32-68 (per expert: ceil(N/32) blocks of ceil(K/256)*8*32 bytes,
    * 16-byte aligned; only w_mx_stride_e is used) */
   int w_mx_layout;
+  /* microscaled activations (MXFP8: x_dtype TAMD_FP8_E4M3 with one e8m0 byte per 32 elements of a row, the
+   * a_mx_scale of matmul.py:131-136): [x_rows, K/32] bytes, unit stride along K/32, indexed by the same (gathered)
+   * row as x; NULL = no block scales.  x_mx_stride_z is the batch pitch. */
+  const uint8_t *x_mx_scale;
+  int64_t x_mx_stride_m, x_mx_stride_z;
 } tamd_matmul_args;
 
 int tamd_matmul(const tamd_matmul_args *args, void *stream);

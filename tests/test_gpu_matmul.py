@@ -541,3 +541,63 @@ def test_ragged_with_preshuffled_scales(block_m, K, N, fp8, device):
                                fused_activation=swiglu_act(1.702, 7.0), c=out_init))
     assert torch.equal(outs[1], outs[0])
     check(outs[1], ref)
+
+
+# ---------------------------------------------------------------------------- MXFP8 activations (block-scaled fp8 rows)
+
+
+def quantize_x_mxfp8(x0, device):
+    """fp32 [.., K] -> (e4m3 values, e8m0 scales per 32 along K) on the GPU, checked against the oracle."""
+    xq, xs = downcast_to_mxfp(x0.to(device), torch.float8_e4m3fn, axis=-1)
+    rq, rs = downcast_to_mxfp_ref(x0, torch.float8_e4m3fn, axis=-1)
+    assert torch.equal(xq.cpu().view(torch.uint8), rq.contiguous().view(torch.uint8)) and torch.equal(xs.cpu(), rs)
+    return xq, xs, rq.contiguous(), rs.contiguous()
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 2048, 512), (16, 64, 64), (33, 96, 208), (130, 192, 528), (70, 2880, 720)])
+@pytest.mark.parametrize("out_dtype", [None, torch.float32])
+def test_mxfp8_activations_dense(M, K, N, out_dtype, device):
+    torch.manual_seed(0)
+    x0 = torch.randn(M, K) * torch.exp(torch.randn(M, K // 32).repeat_interleave(32, dim=1) * 2)  # block-wise dynamic range
+    w = torch.randn(K, N) * 0.02
+    bias = (torch.randn(N) * 0.01).to(torch.bfloat16)
+    v, s, rv, rs = quantize_w(w, device)
+    xq, xs, rq, rxs = quantize_x_mxfp8(x0, device)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32, out_dtype=out_dtype)
+    out = matmul(xq, v, bias.to(device), precision_config=pc)
+    ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, b_mx_scale=rs)
+    assert out.dtype == (out_dtype or torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL * float(ref.float().abs().max()) / 4 + ATOL)
+    # doubling every block scale of the activations doubles the linear part exactly
+    pc32 = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float32)
+    pc32b = PrecisionConfig(a_mx_scale=xs + 1, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float32)
+    assert torch.equal(matmul(xq, v, None, precision_config=pc32b), 2 * matmul(xq, v, None, precision_config=pc32))
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 64, 128])
+@pytest.mark.parametrize("cdna4_scales", [False, True])
+def test_mxfp8_activations_ragged(block_m, cdna4_scales, device):
+    """Gather, scatter with dropped rows, gate weights, SwiGLU; the activation scales follow the gathered rows."""
+    torch.manual_seed(1)
+    E, K, N = 7, 320, 400
+    sizes = torch.tensor([3, 0, 1, 16, 5, 140, 2], dtype=torch.int32)
+    M = int(sizes.sum())
+    x0 = torch.randn(M + 5, K) * torch.exp(torch.randn(M + 5, K // 32).repeat_interleave(32, dim=1))
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    xq, xs, rq, rxs = quantize_x_mxfp8(x0, device)
+    gather = torch.randint(0, M + 5, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::7] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=preshuffle(s) if cdna4_scales else s,
+                         b_microblock_size=32)
+    out_init = torch.zeros((M, N // 2), dtype=torch.bfloat16, device=device)
+    with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+        out = matmul(xq, v, bias.to(device), md, gather_indx=gather.to(device), scatter_indx=scatter.to(device),
+                     precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0), c=out_init)
+    ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, a_mx_scale=rxs,
+                        b_mx_scale=rs, gammas=gammas, fused_swiglu=(1.702, 7.0))
+    check(out, ref)

@@ -48,6 +48,11 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     if (x_rows * a.x_stride_m * esz >= (int64_t)0x7FFFFF00 || (int64_t)a.N * a.w_stride_n >= (int64_t)0x7FFFFF00 ||
         (int64_t)a.N * (cdna4_sc ? (int64_t)(a.K / 32 + 7) : a.w_mx_stride_n) >= (int64_t)0x7FFFFF00)
       return TAMD_E_UNSUPPORTED;
+    if (a.x_mx_scale) {
+      // block scales of the activations: MXFP8 (e4m3 values) through the scaled MFMA only
+      if (!x8) return TAMD_E_UNSUPPORTED;
+      if (a.x_mx_stride_m < a.K / 32 || x_rows * a.x_mx_stride_m >= (int64_t)0x7FFFFF00) return TAMD_E_UNSUPPORTED;
+    }
     int block_m, grid_m;
     if (ragged) {
       block_m = a.block_m;

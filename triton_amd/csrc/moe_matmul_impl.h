@@ -176,6 +176,31 @@ TAMD_DEVICE void dma16(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t so
                  "s"(__builtin_amdgcn_readfirstlane(soff))
                : "memory", "m0");
 }
+// 1-, 2- and 4-byte global -> LDS copies: lane L's value lands (zero-extended) in the dword at
+// lds_addr + 4*L; out-of-range offsets deliver zero.  The five wait states before the load cover an
+// SGPR operand that a v_readfirstlane wrote just before the asm block (the compiler's hazard
+// recognizer does not look inside inline asm) as well as the write of M0.
+TAMD_DEVICE void dma2(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_ushort %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+TAMD_DEVICE void dma1(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_ubyte %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
+TAMD_DEVICE void dma4(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :
+               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
+                 "s"(__builtin_amdgcn_readfirstlane(soff))
+               : "memory", "m0");
+}
 TAMD_DEVICE void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding).
 template <int N>
@@ -381,7 +406,7 @@ TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_
 }
 
 // One output tile with NFR (compile time) active 32-row fragments.
-// LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | e8m0 scales of the tile].
+// LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | (fp8) activation block scales, 2 stages | e8m0 scales of the tile].
 //
 // Both operands reach LDS by DMA.  Activations: 64 K per stage, double buffered; wave w copies rows
 // 8w..8w+7 of every 32-row fragment (8 lanes x 16 B per row); chunk c of row r sits at slot
@@ -411,7 +436,11 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
   const uint32_t lds_b = lds_base + 2 * A_STAGE + wave * 4096;
   const uint8_t *bbuf = lds + 2 * A_STAGE + wave * 4096;
-  uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES;
+  // activation block scales (fp8 path): two stages of four planes (one per 32-K group of the stage) of one dword
+  // per row; a copy always writes 64 dwords (lanes past the tile's rows write zeros)
+  constexpr int AS_ROWS = LDS_ROWS < 64 ? 64 : LDS_ROWS;
+  constexpr int AS_BYTES = FP8 ? 2 * 4 * AS_ROWS * 4 : 0;
+  uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES + AS_BYTES;
 
   // ---- scales of the whole tile, once.  Strided: 256 columns x G bytes, contiguous in memory.  CDNA4
   // pre-shuffle: the tile's 8 blocks of 32 columns are contiguous too (KSP*32 bytes each); byte
@@ -428,7 +457,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       // by DMA, 1 KB per instruction: in flight together with the first activation / weight stages and
       // awaited with them at the first barrier of the K loop
       const v4i_t rs = make_rsrc(sc_src, (uint32_t)sc_avail);
-      const uint32_t lds_sc_addr = lds_base + 2 * A_STAGE + B_BYTES;
+      const uint32_t lds_sc_addr = lds_base + 2 * A_STAGE + B_BYTES + AS_BYTES;
       for (int i = wave; i * 1024 < sc_tile_bytes; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
     } else {
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
@@ -453,6 +482,33 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 
   const int sc_lane_off[2] = {h * (cdna4 ? 64 : 1), (2 + h) * (cdna4 ? 64 : 1)};  // the (2q + h) part of a group's offset
   const int sc_clamp = cdna4 ? 0x7FFFFFFF : G - 1;
+
+  // ---- block scales of the activations (MXFP8): the 4 e8m0 bytes of a row's 128-K stage are copied per stage to
+  // LDS, one byte-sized copy per group (64 rows per instruction, waves 0 and 1; groups past K/32 are not read at
+  // all, so nothing beyond a row's own scales is touched)
+  const bool x_mx = FP8 && a.x_mx_scale != nullptr;
+  const uint32_t lds_as = lds_base + 2 * A_STAGE + B_BYTES;
+  const uint32_t *as_buf = (const uint32_t *)(lds + 2 * A_STAGE + B_BYTES);
+  v4i_t ras = rx;
+  uint32_t as_off = kOob;
+  if (x_mx) {
+    const int64_t xr = a.x_rows > 0 ? a.x_rows : a.M;
+    ras = make_rsrc(a.x_mx_scale + (int64_t)t.z * a.x_mx_stride_z, (uint32_t)(xr * a.x_mx_stride_m));
+    const int r = wave * 64 + lane;
+    if (wave * 64 < LDS_ROWS && r < LDS_ROWS) {
+      const int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
+      const uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
+      as_off = src * (uint32_t)a.x_mx_stride_m;
+    }
+  }
+  auto issue_as = [&](int it) {
+    if (x_mx && wave * 64 < LDS_ROWS) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4)
+        dma1(ras, lds_as + ((it & 1) * 4 + g4) * AS_ROWS * 4 + wave * 256, it * 4 + g4 < G ? as_off : kOob,
+             (uint32_t)(it * 4 + g4));
+    }
+  };
 
   // ---- activation DMA: one instruction per 32-row fragment, lane -> (row 8w + lane/8, slot lane%8)
   const int a_rin = wave * 8 + lane / 8;
@@ -551,6 +607,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       };
       i32x8_t af[2][NFR];
       read_frags(0, af[0]);
+      // A scale operand: lane half h supplies K block h of an MFMA; byte 0 is the group of s = 0, byte 2 of s = 1
+      int sa[NFR];
+#pragma unroll
+      for (int i = 0; i < NFR; ++i)
+        sa[i] = x_mx ? (int)(as_buf[((it & 1) * 4 + h) * AS_ROWS + i * 32 + c32] |
+                             (as_buf[((it & 1) * 4 + 2 + h) * AS_ROWS + i * 32 + c32] << 16))
+                     : 0x7F7F7F7F;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         if (s == 0) read_frags(1, af[1]);
@@ -561,10 +624,10 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
           for (int i = 0; i < NFR; ++i) {
             if (s == 0)
-              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[0][i], bf, acc[i][f], CBSZ, 4, 0, 127, 0,
+              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[0][i], bf, acc[i][f], CBSZ, 4, 0, sa[i], 0,
                                                                         (int)scw[f]);
             else
-              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[1][i], bf, acc[i][f], CBSZ, 4, 0, 127, 1,
+              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[1][i], bf, acc[i][f], CBSZ, 4, 2, sa[i], 1,
                                                                         (int)scw[f]);
           }
         }
@@ -595,11 +658,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   issue_a(0);
   issue_b(0);
   if constexpr (FP8) {
+    issue_as(0);
     for (int it = 0; it < n_ka; ++it) {  // activation and weight stages coincide (128 K each)
       wait_dma();
       __syncthreads();
       load_b(it);
       issue_a(it + 1);
+      issue_as(it + 1);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
       issue_b(it + 1);
       compute(it, std::integral_constant<int, 0>{});
@@ -669,7 +734,7 @@ __global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a,
 template <int XDT, int BM, int ACT>
 int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int LDS_ROWS = TileShape<XDT, BM>::LDS_ROWS;
-  constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES;
+  constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES + (is_fp8(XDT) ? 2 * 4 * (LDS_ROWS < 64 ? 64 : LDS_ROWS) * 4 : 0);
   constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
   int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
   int64_t total = (int64_t)grid_m * grid_n;

@@ -43,25 +43,6 @@ struct Mma16<TAMD_F16> {
   }
 };
 
-// 2- and 4-byte global -> LDS copies: lane L's value lands (zero-extended) in the dword at
-// lds_addr + 4*L; out-of-range offsets deliver zero.  The five wait states before the load cover an
-// SGPR operand that a v_readfirstlane wrote just before the asm block (the compiler's hazard
-// recognizer does not look inside inline asm) as well as the write of M0.
-TAMD_DEVICE void dma2(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_ushort %1, %2, %3 offen lds"
-               :
-               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
-                 "s"(__builtin_amdgcn_readfirstlane(soff))
-               : "memory", "m0");
-}
-TAMD_DEVICE void dma4(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dword %1, %2, %3 offen lds"
-               :
-               : "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(rsrc),
-                 "s"(__builtin_amdgcn_readfirstlane(soff))
-               : "memory", "m0");
-}
-
 // 16-byte copies with an instruction offset: OFF is added to the global offset and to the LDS address
 // alike, so one M0 value serves up to four consecutive 1 KB pieces of a linear image.
 // SETM0: also loads M0 with lds_addr first (with the wait states an SGPR operand written by a

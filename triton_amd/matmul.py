@@ -110,8 +110,14 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         raise NotImplementedError("fused communication needs more than one GPU")
     if c_acc_in is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
         raise NotImplementedError("accumulator input / quantising epilogues are not built")
-    if precision_config.a_mx_scale is not None:
-        raise NotImplementedError("microscaled activations are not built")
+    a_mx_scale = precision_config.a_mx_scale
+    if a_mx_scale is not None:
+        a_mx_scale = _data(a_mx_scale)
+        a_raw = a.storage.data if isinstance(a, Tensor) else a
+        if a_raw.dtype != torch.float8_e4m3fn or a_mx_scale.dtype != torch.uint8:
+            raise NotImplementedError("microscaled activations are built for float8_e4m3fn values with e8m0 scales")
+        mb = precision_config.a_microblock_size
+        assert mb is None or mb == MXFP_BLOCK_SIZE, "Unsupported microscale block size"
     flex = precision_config.flex_ctx
     if flex.acc_data.scale is not None:
         raise NotImplementedError("accumulator flex scale is not built")
@@ -152,7 +158,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     else:
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
-    out_dtype = precision_config.out_dtype or a.dtype
+    # microscaled activations stand for bf16 numbers (the reference dequantises them to bf16, matmul.py:772-778)
+    out_dtype = precision_config.out_dtype or (torch.bfloat16 if a_mx_scale is not None else a.dtype)
     if out_dtype.itemsize == 1 and out_dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f"{out_dtype} outputs are not built (float8_e4m3fn is)")
     rows_out = M
@@ -194,6 +201,13 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     args.x_stride_m = a.stride(-2)
     args.x_stride_z = a.stride(0) if a.ndim == 3 else 0
     args.x_scale = None if flex.lhs_data.scale is None else flex.lhs_data.scale.data_ptr()
+    if a_mx_scale is not None:
+        want = (*a.shape[:-1], K // MXFP_BLOCK_SIZE)
+        assert tuple(a_mx_scale.shape) == want, f"a_mx_scale shape {tuple(a_mx_scale.shape)} != {want}"
+        assert a_mx_scale.stride(-1) == 1 or a_mx_scale.shape[-1] == 1, "a_mx_scale must be contiguous along K"
+        args.x_mx_scale = a_mx_scale.data_ptr()
+        args.x_mx_stride_m = a_mx_scale.stride(-2)
+        args.x_mx_stride_z = a_mx_scale.stride(0) if a_mx_scale.ndim == 3 else 0
     wd = w if w.ndim == 3 else w[None]
     args.w = wd.data_ptr()
     if b.dtype == FP4:
