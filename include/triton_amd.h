@@ -224,6 +224,12 @@ typedef struct tamd_matmul_args {
    * row as x; NULL = no block scales.  x_mx_stride_z is the batch pitch. */
   const uint8_t *x_mx_scale;
   int64_t x_mx_stride_m, x_mx_stride_z;
+  /* MXFP8 output (the quantising epilogue _quantize_mxfp8_fn, mxfp_details/_downcast_to_mxfp.py:218-220): with
+   * y_dtype TAMD_FP8_E4M3 the result is quantised per 32 consecutive output columns of a row exactly as
+   * tamd_downcast_mxfp (ROUND_UP) would quantise the float32 result; the e8m0 bytes go to
+   * y_mx_scale[row, column / 32] (rows placed like the rows of y).  NULL = plain output. */
+  uint8_t *y_mx_scale;
+  int64_t y_mx_stride_m, y_mx_stride_z;
 } tamd_matmul_args;
 
 int tamd_matmul(const tamd_matmul_args *args, void *stream);

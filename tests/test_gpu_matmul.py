@@ -601,3 +601,74 @@ def test_mxfp8_activations_ragged(block_m, cdna4_scales, device):
     ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, a_mx_scale=rxs,
                         b_mx_scale=rs, gammas=gammas, fused_swiglu=(1.702, 7.0))
     check(out, ref)
+
+
+# ---------------------------------------------------------------------------- MXFP8 output (quantising epilogue)
+
+
+def mxfp8_epilogue():
+    from triton_amd.matmul import Epilogue
+    return Epilogue(FnSpecs("QUANTIZE_MXFP8", None, (), ()), tuple(), tuple(), effective_itemsize=6.0)
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 2048, 512), (16, 64, 64), (33, 96, 208), (130, 192, 528)])
+@pytest.mark.parametrize("act", [False, True])
+def test_mxfp8_output_dense(M, K, N, act, device):
+    """The quantised result must be bit for bit what downcast_to_mxfp makes of the float32 result of the same kernel
+    (values and scale bytes), and dequantise to the oracle's result within the fp8 step."""
+    torch.manual_seed(0)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(K, N) * 0.02
+    bias = torch.randn(N)
+    v, s, rv, rs = quantize_w(w, device)
+    fa = swiglu_act(1.702, 7.0) if act else None
+    n_out = N // 2 if act else N
+    y32 = matmul(x.to(device), v, bias.to(device), fused_activation=fa,
+                 precision_config=PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float32))
+    c_scale = torch.zeros((M, -(-n_out // 32)), dtype=torch.uint8, device=device)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, c_mx_scale=c_scale)
+    yq = matmul(x.to(device), v, bias.to(device), fused_activation=fa, precision_config=pc, epilogue=mxfp8_epilogue())
+    assert yq.dtype == torch.float8_e4m3fn and tuple(yq.shape) == (M, n_out) and pc.c_microblock_size == 32
+    pad = (-n_out) % 32
+    y32p = torch.nn.functional.pad(y32.cpu(), (0, pad))
+    want_v, want_s = downcast_to_mxfp_ref(y32p, torch.float8_e4m3fn, axis=-1)
+    assert torch.equal(c_scale.cpu(), want_s)
+    assert torch.equal(yq.cpu().view(torch.uint8), want_v[:, :n_out].contiguous().view(torch.uint8))
+    ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs, fused_swiglu=(1.702, 7.0) if act else None).float()
+    from oracle.mxfp_ref import upcast_from_mxfp_ref
+    deq = upcast_from_mxfp_ref(torch.nn.functional.pad(yq.cpu().view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn),
+                               c_scale.cpu(), torch.float32, axis=-1)[:, :n_out]
+    gmax = torch.nn.functional.pad(ref.abs(), (0, pad)).reshape(M, -1, 32).amax(dim=-1).repeat_interleave(32, dim=1)[:, :n_out]
+    assert torch.all((deq - ref).abs() <= gmax / 8 + 2e-2)  # e4m3 step at the top of a group is 1/16 of its maximum
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 128])
+def test_mxfp8_output_ragged_then_mxfp8_input(block_m, device):
+    """FC1 (SwiGLU, MXFP8 output, expert-sorted rows) feeding FC2 as MXFP8 activations (scattered, gate weights)."""
+    torch.manual_seed(1)
+    E, K, N = 7, 320, 448
+    sizes = torch.tensor([3, 0, 1, 16, 5, 140, 2], dtype=torch.int32)
+    M = int(sizes.sum())
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w1 = torch.randn(E, K, N) * 0.05
+    w2 = torch.randn(E, N // 2, 256) * 0.05
+    b1, b2 = torch.randn(E, N), torch.randn(E, 256)
+    v1, s1, rv1, rs1 = quantize_w(w1, device)
+    v2, s2, rv2, rs2 = quantize_w(w2, device)
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    scatter = torch.randperm(M, dtype=torch.int32)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    h_scale = torch.zeros((M, N // 2 // 32), dtype=torch.uint8, device=device)
+    pc1 = PrecisionConfig(b_mx_scale=s1, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, c_mx_scale=h_scale)
+    with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+        h = matmul(x.to(device), v1, b1.to(device), md, precision_config=pc1, fused_activation=swiglu_act(1.702, 7.0),
+                   epilogue=mxfp8_epilogue())
+        h32 = matmul(x.to(device), v1, b1.to(device), md, fused_activation=swiglu_act(1.702, 7.0),
+                     precision_config=PrecisionConfig(b_mx_scale=s1, b_microblock_size=32, out_dtype=torch.float32))
+        want_v, want_s = downcast_to_mxfp_ref(h32.cpu(), torch.float8_e4m3fn, axis=-1)
+        assert torch.equal(h_scale.cpu(), want_s) and torch.equal(h.cpu().view(torch.uint8), want_v.contiguous().view(torch.uint8))
+        pc2 = PrecisionConfig(a_mx_scale=h_scale, a_microblock_size=32, b_mx_scale=s2, b_microblock_size=32)
+        y = matmul(h, v2, b2.to(device), md, scatter_indx=scatter.to(device), precision_config=pc2, gammas=gammas.to(device))
+    ref = MR.matmul_ref(want_v.contiguous(), rv2, b2, slice_sizes=sizes, scatter_indx=scatter, a_mx_scale=want_s,
+                        b_mx_scale=rs2, gammas=gammas)
+    check(y, ref)

@@ -53,6 +53,7 @@ class MatmulArgs(C.Structure):
         ("y_expected_scale", C.c_void_p), ("y_actual_scale", C.c_void_p), ("y_saturate_inf", C.c_int),
         ("w_mx_layout", C.c_int),
         ("x_mx_scale", C.c_void_p), ("x_mx_stride_m", C.c_int64), ("x_mx_stride_z", C.c_int64),
+        ("y_mx_scale", C.c_void_p), ("y_mx_stride_m", C.c_int64), ("y_mx_stride_z", C.c_int64),
     ]
 
 

@@ -308,6 +308,30 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
         for (int p = 0; p < NO; ++p) o[p] *= gamma;
       }
       if constexpr (FLEX) {
+        if (a.y_mx_scale) {
+          // MXFP8 output: a group is 32 consecutive output columns of a row = the outputs of one half wave (of
+          // half of it when a lane holds two columns).  max |o| over the group, scale = 2^ceil(log2(max / 448)),
+          // o / scale clamped to +-448; the cast below rounds to nearest even (as tamd_downcast_mxfp does).
+          float m = 0.f;
+#pragma unroll
+          for (int p = 0; p < NO; ++p) m = __builtin_fmaxf(m, out_col0 + p < n_out ? __builtin_fabsf(o[p]) : 0.f);
+#pragma unroll
+          for (int sh = 16 / NO; sh > 0; sh >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, sh));
+          const uint32_t sb = (f32_to_bits(m / 448.0f) + 0x007FFFFFu) & 0x7F800000u;
+          const float ds = bits_to_f32(sb);
+          const float qs = ds == 0.f ? 0.f : 1.0f / ds;
+#pragma unroll
+          for (int p = 0; p < NO; ++p) {
+            const float q = o[p] * qs;
+            o[p] = q != q ? q : __builtin_fminf(__builtin_fmaxf(q, -448.0f), 448.0f);
+          }
+          // one lane per group stores the scale byte (the row may be scattered or dropped)
+          if ((c32 & (32 / NO - 1)) == 0 && r < t.rows && out_col0 < n_out) {
+            int64_t dst = t.start_m + t.off_m + r;
+            if (a.scatter_indx) dst = a.scatter_indx[dst];
+            if (dst >= 0) a.y_mx_scale[(int64_t)t.z * a.y_mx_stride_z + dst * a.y_mx_stride_m + out_col0 / 32] = (uint8_t)(sb >> 23);
+          }
+        }
         if (track_max && r < t.rows) {
 #pragma unroll
           for (int p = 0; p < NO; ++p)

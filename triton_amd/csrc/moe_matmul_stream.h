@@ -422,6 +422,7 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   if (a.bias && !aligned(a.bias, a.bias_dtype == TAMD_F32 ? 4 : 2)) return false;
   if (a.N % 16 != 0) return false;  // whole 16-column groups only (their scale run is then a multiple of 16 bytes)
   if (a.block_schedule && !a.block_offs) return false;
+  if (a.y_mx_scale) return false;  // a unit is 16 columns, an output scale group 32
   return true;
 }
 

@@ -108,8 +108,19 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         raise NotImplementedError("K-ragged matmul is not built for gfx950")
     if fused_comm is not None:
         raise NotImplementedError("fused communication needs more than one GPU")
-    if c_acc_in is not None or epilogue.specs.name != "dflt" or precision_config.c_mx_scale is not None:
-        raise NotImplementedError("accumulator input / quantising epilogues are not built")
+    if c_acc_in is not None:
+        raise NotImplementedError("accumulator input is not built")
+    # quantising epilogue: MXFP8 (float8_e4m3fn values, e8m0 scale per 32 output columns), tests/test_matmul.py:547-561
+    c_mx_scale = precision_config.c_mx_scale
+    mx_out = c_mx_scale is not None
+    if epilogue.specs.name.lower() not in ("dflt", "quantize_mxfp8") or (epilogue.specs.name != "dflt") != mx_out:
+        raise NotImplementedError(f"epilogue {epilogue.specs.name!r} / c_mx_scale combination is not built (MXFP8 is)")
+    if mx_out:
+        c_mx_scale = _data(c_mx_scale)
+        if c_mx_scale.dtype != torch.uint8 or (precision_config.c_microblock_size or MXFP_BLOCK_SIZE) != MXFP_BLOCK_SIZE:
+            raise NotImplementedError("output scales are built as e8m0 bytes per 32 columns")
+        precision_config.c_microblock_size = MXFP_BLOCK_SIZE
+        precision_config.c_value_pack_factor = 1
     a_mx_scale = precision_config.a_mx_scale
     if a_mx_scale is not None:
         a_mx_scale = _data(a_mx_scale)
@@ -160,6 +171,12 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     red_n = fused_activation.specs.reduction_n
     # microscaled activations stand for bf16 numbers (the reference dequantises them to bf16, matmul.py:772-778)
     out_dtype = precision_config.out_dtype or (torch.bfloat16 if a_mx_scale is not None else a.dtype)
+    if mx_out:
+        out_dtype = precision_config.out_dtype or (c.dtype if c is not None else torch.float8_e4m3fn)
+        if out_dtype != torch.float8_e4m3fn:
+            raise NotImplementedError("MXFP8 output needs float8_e4m3fn values")
+        if flex.out_data.expected_scale is not None or flex.out_data.actual_scale is not None:
+            raise NotImplementedError("flexpoint output scales together with MX output scales are not built")
     if out_dtype.itemsize == 1 and out_dtype != torch.float8_e4m3fn:
         raise NotImplementedError(f"{out_dtype} outputs are not built (float8_e4m3fn is)")
     rows_out = M
@@ -264,6 +281,13 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if flex.out_data.actual_scale is not None:
         args.y_actual_scale = flex.out_data.actual_scale.data_ptr()
     args.y_saturate_inf = int(precision_config.flexpoint_saturate_inf)
+    if mx_out:
+        n_groups = -(-(N // red_n) // MXFP_BLOCK_SIZE)
+        cs = c_mx_scale if c_mx_scale.ndim == 3 else c_mx_scale[None]
+        assert tuple(cs.shape) == (batch, rows_out, n_groups), \
+            f"c_mx_scale shape {tuple(c_mx_scale.shape)} != {(rows_out, n_groups)}"
+        assert cs.stride(-1) == 1 or cs.shape[-1] == 1, "c_mx_scale must be contiguous along its last axis"
+        args.y_mx_scale, args.y_mx_stride_m, args.y_mx_stride_z = cs.data_ptr(), cs.stride(1), cs.stride(0)
     args.gather_indx, args.scatter_indx = i32(gather_indx), i32(scatter_indx)
     if ragged:
         md = a_ragged_metadata
