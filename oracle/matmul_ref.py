@@ -113,3 +113,23 @@ def reduce_ref(x: torch.Tensor, dim: int, mask=None, scale=None):
     if mask is not None:
         xf = torch.where(mask.to(torch.bool), xf, torch.zeros((), dtype=torch.float32))
     return xf.sum(dim=dim).to(x.dtype)
+
+
+def reduce_mx_ref(x: torch.Tensor, x_mxscale: torch.Tensor, dim: int, mask=None, scale=None, x_flex_scale=None):
+    """The microscaled branch of reduce_torch (reduce.py:1185-1206): dequantise x (fp8 values, e8m0 scales along the
+    last axis) to float32, masked / scaled sum over `dim`, quantise the float32 result to MXFP8 along the last axis.
+    The sum runs in index order r = 0, 1, ... (one float32 addition per step), which fixes the rounding the GPU kernel
+    has to reproduce.  Returns (values float8_e4m3fn, scales uint8)."""
+    from .mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+    xf = upcast_from_mxfp_ref(x, x_mxscale, torch.float32, axis=-1)
+    if x_flex_scale is not None:
+        xf = xf * x_flex_scale.to(torch.float32)
+    if scale is not None:
+        xf = xf * scale.to(torch.float32)
+    if mask is not None:
+        xf = torch.where(mask.to(torch.bool), xf, torch.zeros((), dtype=torch.float32))
+    dim = dim % xf.ndim
+    acc = torch.zeros([n for i, n in enumerate(xf.shape) if i != dim], dtype=torch.float32)
+    for r in range(xf.shape[dim]):
+        acc = acc + xf.select(dim, r)
+    return downcast_to_mxfp_ref(acc, torch.float8_e4m3fn, axis=-1)

@@ -47,3 +47,31 @@ def test_swiglu(M, N, limit, dtype, device):
     ref = MR.swiglu_ref(x, 0.5, limit)
     tol = dict(rtol=1e-2, atol=1e-2) if dtype != torch.float32 else dict(rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(out.cpu().float(), ref.float(), **tol)
+
+
+@pytest.mark.parametrize("shape,dim", [((64, 4, 256), 1), ((4, 40, 96), 0), ((37, 5, 64), 1)])
+@pytest.mark.parametrize("mask_mode", [None, "broadcast_last"])
+@pytest.mark.parametrize("use_scale,use_flex", [(False, False), (True, False), (True, True)])
+def test_reduce_mxfp8_in_and_out(shape, dim, mask_mode, use_scale, use_flex, device):
+    """Microscaled branch: fp8 values + e8m0 scales along the last axis in, the same out; bit-exact against the oracle
+    (which adds in index order, as the kernel does)."""
+    from oracle.mxfp_ref import downcast_to_mxfp_ref
+    from triton_amd.numerics import InFlexData
+    torch.manual_seed(0)
+    x0 = torch.randn(shape) * torch.exp(torch.randn(shape[:-1] + (1, )))
+    xv, xs = downcast_to_mxfp_ref(x0, torch.float8_e4m3fn, axis=-1)
+    xv, xs = xv.contiguous(), xs.contiguous()
+    mask = None
+    if mask_mode == "broadcast_last":
+        mask = torch.rand(shape[:-1] + (1, )) > 0.3
+    sshape = [1] * len(shape)
+    sshape[dim] = shape[dim]
+    scale = torch.rand(sshape) + 0.5 if use_scale else None
+    fscale = torch.tensor([0.75]) if use_flex else None
+    yv, ys = reduce(xv.to(device), dim, mask=None if mask is None else mask.to(device),
+                    scale=None if scale is None else scale.to(device), x_mxscale=xs.to(device),
+                    x_flex=InFlexData(dtype=torch.float8_e4m3fn, scale=fscale.to(device)) if use_flex else InFlexData())
+    rv, rs = MR.reduce_mx_ref(xv, xs, dim, mask=mask, scale=None if scale is None else (scale * 0.75 if use_flex else scale),
+                              x_flex_scale=None)
+    assert yv.dtype == torch.float8_e4m3fn and torch.equal(ys.cpu(), rs)
+    assert torch.equal(yv.cpu().view(torch.uint8), rv.contiguous().view(torch.uint8))

@@ -155,3 +155,22 @@ def test_reduce_direct_sum():
                     acc = np.float32(acc + np.float32(float(x[t, j, n])) * np.float32(float(scale[t, j, 0])))
             assert float(z[t, n]) == float(torch.tensor(float(acc)).bfloat16()), (t, n)
     assert torch.equal(MR.reduce_ref(x, 1), x.float().sum(1).bfloat16())
+
+
+def test_reduce_mx_small_integers_by_hand():
+    """reduce.py:1185-1206: dequantise, sum over `dim`, quantise to MXFP8.  With small integers every step is exact,
+    so the result must be the MXFP8 image of the plain integer sum."""
+    from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+    torch.manual_seed(3)
+    x = torch.randint(-6, 7, (5, 3, 64)).float()
+    xv, xs = downcast_to_mxfp_ref(x, torch.float8_e4m3fn, axis=-1)
+    assert torch.equal(upcast_from_mxfp_ref(xv, xs, torch.float32, axis=-1), x)  # small integers survive MXFP8
+    mask = torch.tensor([True, False, True]).reshape(1, 3, 1)
+    scale = torch.tensor([2.0, 4.0, 0.5]).reshape(1, 3, 1)
+    yv, ys = MR.reduce_mx_ref(xv.contiguous(), xs.contiguous(), 1, mask=mask, scale=scale)
+    want = 2.0 * x[:, 0] + 0.5 * x[:, 2]
+    wv, ws = downcast_to_mxfp_ref(want, torch.float8_e4m3fn, axis=-1)
+    assert torch.equal(ys, ws) and torch.equal(yv.contiguous().view(torch.uint8), wv.contiguous().view(torch.uint8))
+    for t in range(5):  # and that image is within half an fp8 step of the exact sum
+        got = upcast_from_mxfp_ref(yv, ys, torch.float32, axis=-1)[t]
+        assert torch.all((got - want[t]).abs() <= want[t].abs().reshape(2, 32).amax(dim=1).repeat_interleave(32) / 16 + 1e-6)

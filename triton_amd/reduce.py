@@ -28,11 +28,29 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
     in float32 in index order and cast to y_dtype (default x.dtype)."""
     def _flex_used(f):
         return f is not None and any(getattr(f, n, None) is not None for n in ("scale", "expected_scale", "actual_scale"))
-    if x_mxscale is not None or y_has_mx or _flex_used(x_flex) or _flex_used(y_flex) or x_global_scale is not None \
-            or postprocess_fn1 is not None or postprocess_fn2 is not None or unpadded_batch_size is not None:
-        raise NotImplementedError("mx / flex / postprocess variants of reduce are not built")
+    if _flex_used(y_flex) or x_global_scale is not None or postprocess_fn1 is not None or postprocess_fn2 is not None \
+            or unpadded_batch_size is not None:
+        raise NotImplementedError("output flex / global scale / postprocess variants of reduce are not built")
     _lib.require_gpu(x, "x")
     dim = dim % x.ndim
+    x_flex_scale = getattr(x_flex, "scale", None) if x_flex is not None else None
+    if x_flex_scale is not None:
+        # one float32 factor on the input: folded into the per-element scale operand
+        fs = x_flex_scale.to(torch.float32).reshape((1, ) * x.ndim)
+        scale = fs if scale is None else scale.to(torch.float32) * fs
+    if x_mxscale is not None:
+        # microscaled input and output (reduce.py:1185-1206 of the reference): dequantise along the last axis, sum in
+        # float32, quantise the sum to MXFP8 along the last axis -- three launches of the kernels of this library
+        from .numerics_details.mxfp import downcast_to_mxfp, upcast_from_mxfp
+        assert dim != x.ndim - 1, "the microscaled axis cannot be reduced"
+        assert y is None and y_has_mx in (None, True) and y_microblock_size == 32 and y_value_pack_factor == 1
+        x32 = upcast_from_mxfp(x, x_mxscale, torch.float32, axis=-1)
+        y32, _ = reduce(x32, dim, mask=mask, scale=scale, y_dtype=torch.float32)
+        return downcast_to_mxfp(y32, torch.float8_e4m3fn, axis=-1)
+    if y_has_mx:
+        raise NotImplementedError("a microscaled output needs a microscaled input (as in the reference's torch twin)")
+    if x.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        raise NotImplementedError("fp8 inputs without block scales are not built")
     lead = 1
     for s in x.shape[:dim]:
         lead *= s
