@@ -35,6 +35,8 @@ WORKLOADS = {
     "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
     # down projection + combine: fp8 (per-tensor scaled) expert-sorted rows x MXFP4 W2, gate weights, scatter, k-way sum
     "fc2_combine": dict(T=16384, E=32, k=4, K=2880, N=2880, act=False, fc2=True),
+    # the down projection at decode size (fp8 rows of 64 tokens): weight streaming through the tiled fp8 kernel
+    "fc2_decode": dict(T=64, E=128, k=4, K=2880, N=2880, act=False, fc2=True),
     # BASELINE config 1: one dense bf16 x MXFP4 product with bias (launch / latency bound: 7.6 MB, 4.3 GFLOP)
     "c1_dense": dict(M=256, K=2048, N=4096, dense=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
@@ -237,11 +239,18 @@ def run_fc2(args, cfg):
     n_active = int((col_sum > 0).sum())
     mm_bytes = rows * K + n_active * (K // 2 * N + K // 32 * N + N * 2) + rows * 8 + rows * N * 2
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
-    roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_FP8_TFLOPS, unit="TFLOP/s",
-                frac=round(tflops_kernel / PEAK_FP8_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
-                kernel="mm_x8_mxfp4_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
-                algorithmic_flops=flops, frac_of_mxfp4_peak=round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4),
-                hbm_gbs=round(mm_bytes / (kernel_ms * 1e-3) / 1e9, 1))
+    gbs_kernel = mm_bytes / (kernel_ms * 1e-3) / 1e9
+    if rows <= 16 * E:  # decode size: weight streaming, bound by HBM
+        roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
+                    kernel="mm_stream16_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
+                    algorithmic_flops=flops)
+    else:
+        roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_FP8_TFLOPS, unit="TFLOP/s",
+                    frac=round(tflops_kernel / PEAK_FP8_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
+                    kernel="mm_x8_mxfp4_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
+                    algorithmic_flops=flops, frac_of_mxfp4_peak=round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4),
+                    hbm_gbs=round(gbs_kernel, 1))
     ref = RR.routing_ref(logits_cpu, k)
     routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(col_sum, ref["col_sum"]))
     gam_ref = ref["vals"].flatten()[ref["col_sorted_indx"].long()]

@@ -672,3 +672,41 @@ def test_mxfp8_output_ragged_then_mxfp8_input(block_m, device):
     ref = MR.matmul_ref(want_v.contiguous(), rv2, b2, slice_sizes=sizes, scatter_indx=scatter, a_mx_scale=want_s,
                         b_mx_scale=rs2, gammas=gammas)
     check(y, ref)
+
+
+@pytest.mark.parametrize("K", [64, 1024, 2880, 4096])
+@pytest.mark.parametrize("mx", [False, True])
+@pytest.mark.parametrize("act", [False, True])
+def test_decode_row_blocks_of_16_fp8_rows(K, mx, act, device):
+    """The streaming kernel with float8_e4m3fn rows (per-tensor flex scale, or MXFP8 block scales), expanded to bf16
+    as a row block is loaded; gather, scatter with dropped rows, gate weights."""
+    torch.manual_seed(K)
+    E, N = 7, 608
+    sizes = torch.tensor([3, 0, 1, 16, 5, 21, 2], dtype=torch.int32)
+    M = int(sizes.sum())
+    x0 = torch.randn(M + 5, K) * torch.exp(torch.randn(M + 5, K // 32).repeat_interleave(32, dim=1))
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    gather = torch.randint(0, M + 5, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::7] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    kw = dict(slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs, gammas=gammas,
+              fused_swiglu=(1.702, 7.0) if act else None)
+    if mx:
+        xq, xs, rq, rxs = quantize_x_mxfp8(x0, device)
+        pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32)
+        ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, **kw)
+    else:
+        x8, x_scale = to_fp8(x0)
+        xq = x8.to(device)
+        pc = fp8_pc(s, x_scale, device, torch.bfloat16)
+        ref = MR.matmul_ref(x8, rv, bias, a_flex_scale=x_scale, **kw).to(torch.bfloat16)
+    out_init = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=device)
+    with scoped_opt_flags_constraints({"block_m": 16}):
+        out = matmul(xq, v, bias.to(device), md, gather_indx=gather.to(device), scatter_indx=scatter.to(device),
+                     precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0) if act else None,
+                     c=out_init)
+    check(out, ref)

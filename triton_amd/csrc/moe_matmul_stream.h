@@ -82,7 +82,9 @@ struct StreamShape {
 // issue and await the copies, waves 6-7 finish and store the previous unit.  A wave that issues copies
 // stalls whenever the memory pipeline is full; with nothing else to do it refills the pipeline the
 // moment there is room, and the stalls never delay MFMA work or stores.
-template <int XDT, int ACT, int SS, int RING>
+// A8: the activations are stored as float8_e4m3fn (optionally with e8m0 block scales per 32 K) and are expanded to
+// XDT when a row block's slice is loaded into registers -- exact, so the K loop is the same as for 16-bit rows.
+template <int XDT, int ACT, int SS, int RING, bool A8>
 __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
@@ -345,15 +347,43 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       int rc = c16 < cb.rows ? c16 : cb.rows - 1;
       rc = cb.row0 + (rc < 0 ? 0 : rc);
       const int64_t src = a.gather_indx ? (int64_t)a.gather_indx[rc] : (int64_t)rc;
-      const uint16_t *xr = (const uint16_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+      if constexpr (A8) {
+        const uint8_t *xr = (const uint8_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+        const uint8_t *xs = a.x_mx_scale ? a.x_mx_scale + (int64_t)cb.z * a.x_mx_stride_z + src * a.x_mx_stride_m : nullptr;
 #pragma unroll
-      for (int j = 0; j < SS; ++j) {
-        const int kg = kb + 4 * j + g;
+        for (int j = 0; j < SS; ++j) {
+          const int kg = kb + 4 * j + g;
+          const bool live = kg < G && cb.rows > 0;
+          const float mult = (live && xs) ? bits_to_f32((uint32_t)xs[kg] << 23) : 1.0f;  // 2^(e - 127); 0xFF gives +inf
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          uint4 v = make_uint4(0, 0, 0, 0);
-          if (kg < G && cb.rows > 0) v = *(const uint4 *)(xr + 32 * kg + 8 * u);
-          areg[j * 4 + u] = __builtin_bit_cast(frag_t, v);
+          for (int u = 0; u < 4; ++u) {
+            uint2 v = make_uint2(0, 0);
+            if (live) v = *(const uint2 *)(xr + 32 * kg + 8 * u);
+            float f[8];
+            f[0] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 0) * mult;
+            f[1] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 1) * mult;
+            f[2] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 2) * mult;
+            f[3] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 3) * mult;
+            f[4] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 0) * mult;
+            f[5] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 1) * mult;
+            f[6] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 2) * mult;
+            f[7] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 3) * mult;
+            typedef decltype(frag_t{}[0]) elem_t;
+            areg[j * 4 + u] = frag_t{(elem_t)f[0], (elem_t)f[1], (elem_t)f[2], (elem_t)f[3],
+                                     (elem_t)f[4], (elem_t)f[5], (elem_t)f[6], (elem_t)f[7]};
+          }
+        }
+      } else {
+        const uint16_t *xr = (const uint16_t *)a.x + (int64_t)cb.z * a.x_stride_z + src * a.x_stride_m;
+#pragma unroll
+        for (int j = 0; j < SS; ++j) {
+          const int kg = kb + 4 * j + g;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (kg < G && cb.rows > 0) v = *(const uint4 *)(xr + 32 * kg + 8 * u);
+            areg[j * 4 + u] = __builtin_bit_cast(frag_t, v);
+          }
         }
       }
     };
@@ -426,7 +456,7 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   return true;
 }
 
-template <int XDT, int ACT, int SS>
+template <int XDT, int ACT, int SS, bool A8>
 int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + (SS + 1) / 2 * 1024 + 256);
   constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
@@ -438,20 +468,20 @@ int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (e != hipSuccess) return (int)e;
   const int wgs = (int)(upper < cus ? upper : cus);
-  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING>;
+  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, A8>;
   e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
   if (e != hipSuccess) return (int)e;
   kern<<<dim3((unsigned)wgs), 512, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
   return launch_status();
 }
 
-template <int XDT, int ACT>
+template <int XDT, int ACT, bool A8 = false>
 int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int ss = (a.K / 32 + 15) / 16;  // super steps per wave
-  if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2>(a, grid_m, st);
-  if (ss <= 4) return launch_stream16_ss<XDT, ACT, 4>(a, grid_m, st);
-  if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6>(a, grid_m, st);
-  return launch_stream16_ss<XDT, ACT, 8>(a, grid_m, st);
+  if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2, A8>(a, grid_m, st);
+  if (ss <= 4) return launch_stream16_ss<XDT, ACT, 4, A8>(a, grid_m, st);
+  if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6, A8>(a, grid_m, st);
+  return launch_stream16_ss<XDT, ACT, 8, A8>(a, grid_m, st);
 }
 
 }  // namespace tamd
