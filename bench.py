@@ -35,6 +35,9 @@ WORKLOADS = {
     "fc1_prefill_e8": dict(T=4096, E=8, k=4, K=2880, N=5760, act=True),
     # down projection + combine: fp8 (per-tensor scaled) expert-sorted rows x MXFP4 W2, gate weights, scatter, k-way sum
     "fc2_combine": dict(T=16384, E=32, k=4, K=2880, N=2880, act=False, fc2=True),
+    # fc1_prefill with the activations quantised to MXFP8 inside the step (downcast_to_mxfp + scaled-MFMA matmul):
+    # the block-scaled fp8 x fp4 path of the hardware; NOT interchangeable with the bf16 workload (x loses precision)
+    "fc1_prefill_mx8": dict(T=4096, E=128, k=4, K=2880, N=5760, act=True, mx8=True),
     # the down projection at decode size (fp8 rows of 64 tokens): weight streaming through the tiled fp8 kernel
     "fc2_decode": dict(T=64, E=128, k=4, K=2880, N=2880, act=False, fc2=True),
     # BASELINE config 1: one dense bf16 x MXFP4 product with bias (launch / latency bound: 7.6 MB, 4.3 GFLOP)
@@ -335,11 +338,21 @@ def main():
     fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if act else None
     constraints = {"block_m": args.block_m} if args.block_m else {}
 
+    mx8 = bool(cfg.get("mx8"))
+    if mx8:
+        from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+
     def step(ev=None):
         r = routing(logits, k)
+        if mx8:
+            xq, xs = downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
+            pcs = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=pc.b_mx_scale, b_microblock_size=32)
         if ev is not None:
             ev[0].record()
-        y = matmul(x, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=fa)
+        if mx8:
+            y = matmul(xq, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pcs, fused_activation=fa)
+        else:
+            y = matmul(x, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=fa)
         if ev is not None:
             ev[1].record()
         return r, y
@@ -368,15 +381,16 @@ def main():
     tflops_step = flops / (ms_per_step * 1e-3) / 1e12
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
     gbs_kernel = abytes / (kernel_ms * 1e-3) / 1e9
-    hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (PEAK_BF16_TFLOPS * 1e12))
+    peak_mfma = PEAK_FP8_TFLOPS if mx8 else PEAK_BF16_TFLOPS
+    hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (peak_mfma * 1e12))
     if hbm_bound:
         roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                     frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
     else:
-        roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                    frac=round(tflops_kernel / PEAK_BF16_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
+        roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=peak_mfma, unit="TFLOP/s",
+                    frac=round(tflops_kernel / peak_mfma, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
     # row blocks of 16 (few rows per expert) run the weight-streaming kernel, everything else the tiled one
-    roof["kernel"] = "mm_stream16_kernel" if rows <= 16 * E else "mm_x16_mxfp4_kernel"
+    roof["kernel"] = "mm_stream16_kernel" if rows <= 16 * E else ("mm_x8_mxfp4_kernel" if mx8 else "mm_x16_mxfp4_kernel")
     roof["kernel_ms"] = round(kernel_ms, 4)
     roof["algorithmic_bytes"] = abytes
     roof["algorithmic_flops"] = flops
@@ -391,7 +405,12 @@ def main():
     gemm_ok = None
     if args.cpu_experts > 0:
         n_e = min(args.cpu_experts, E)
-        y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, n_e, K, N, act)
+        x_ref = x_cpu
+        if mx8:  # the oracle sees the same quantised activations, dequantised (exactly) to bf16
+            from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+            qv, qs = downcast_to_mxfp_ref(x_cpu, torch.float8_e4m3fn, axis=-1)
+            x_ref = upcast_from_mxfp_ref(qv, qs, torch.bfloat16, axis=-1)
+        y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x_ref, vals, scales, bias_cpu, ref, n_e, K, N, act)
         gemm_ok = bool(torch.allclose(y[:n_rows].cpu().float(), y_ref.float(), rtol=1e-2, atol=1e-2))
         cpu = dict(value=round(cpu_tflops, 5), unit="TFLOP/s", cores=os.cpu_count(), kind="port",
                    sample=f"oracle matmul_ref (dequantise + fp32 GEMM + SwiGLU) on the first {n_e} of {E} experts "
@@ -399,8 +418,10 @@ def main():
     out = {
         "metric": "moe_matmul_ogs_tflops", "value": round(tflops_step, 2), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x mxfp4 (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: routing + matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, "
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": ("mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") + " (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: routing + " + ("downcast_to_mxfp(x) + " if mx8 else "") +
+                               f"matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, "
                                f"hidden={K}, experts={E}, top-{k}, W1 mxfp4 [{E},{K},{N}]",
                    "rows": rows, "active_experts": n_active, "scale_layout": args.scale_layout},
         "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),

@@ -136,3 +136,17 @@ def test_errors_before_launch():
         matmul(torch.zeros(2, 4, 64), torch.zeros(2, 64, 8), None, gather_indx=torch.zeros(4, dtype=torch.int32))
     with pytest.raises((RuntimeError, NotImplementedError)):
         matmul(x, w, None)  # CPU tensors: no CPU path exists
+
+
+def test_build_reports_kernels_in_scratch_memory():
+    # the build refuses a kernel that fell out of registers: it would still be right, and several times slower
+    from triton_amd.build import _scratch_users
+    remarks = """
+x.h:1:1: remark: Function Name: _ZN4tamd1aEv [-Rpass-analysis=kernel-resource-usage]
+x.h:1:1: remark:     VGPRs: 242 [-Rpass-analysis=kernel-resource-usage]
+x.h:1:1: remark:     ScratchSize [bytes/lane]: 704 [-Rpass-analysis=kernel-resource-usage]
+x.h:9:1: remark: Function Name: _ZN4tamd1bEv [-Rpass-analysis=kernel-resource-usage]
+x.h:9:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+"""
+    assert _scratch_users(remarks) == [("_ZN4tamd1aEv", 704)]
+    assert _scratch_users("") == []

@@ -3,6 +3,7 @@
 Usage: python -m triton_amd.build [--force]
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -11,21 +12,46 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtriton_amd.so")
 SOURCES = ["api.cpp", "mxfp.hip", "routing.hip", "elementwise.hip", "moe_matmul.hip", "moe_matmul_bf16.hip", "moe_matmul_f16.hip",
-           "moe_matmul_fp8.hip"]
+           "moe_matmul_fp8.hip", "moe_matmul_stream_bf16.hip", "moe_matmul_stream_f16.hip", "moe_matmul_stream_fp8.hip",
+           "moe_matmul_w16_bf16.hip", "moe_matmul_w16_f16.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-# packed fp32 math is switched off on purpose (device code only)
+# packed fp32 math is switched off on purpose (device code only); the unroll limit is raised because the tile
+# epilogues index their accumulators with loops that must unroll completely (up to 80 element rows per lane):
+# at the default limit the largest ones stay rolled and the accumulators drop into scratch memory
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-packed-fp32-ops", "-mllvm", "-pragma-unroll-threshold=65536", "-Wno-unused-command-line-argument"]
 
 
 EXTRA = os.environ.get("TAMD_EXTRA_HIPCC_FLAGS", "").split()  # e.g. -DTAMD_STREAM_WGS_PER_CU=1 for experiments
 
 
+def _scratch_users(remarks):
+    """Kernels that use scratch memory (register spills or arrays the compiler could not keep in registers),
+    from the kernel-resource-usage remarks: [(mangled name, bytes per lane)]."""
+    out, name = [], None
+    for line in remarks.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and int(m.group(1)) > 0:
+            out.append((name, int(m.group(1))))
+    return out
+
+
 def _compile(src, obj):
     cmd = [HIPCC, *FLAGS, *EXTRA, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+    if src.endswith(".hip"):
+        cmd.append("-Rpass-analysis=kernel-resource-usage")
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{res.stdout}\n{res.stderr}")
+    # every kernel here is written to live in registers; one that falls into scratch memory still computes
+    # the right values, several times slower, so the build is where it has to be caught
+    spilled = _scratch_users(res.stderr)
+    if spilled and not os.environ.get("TAMD_ALLOW_SCRATCH"):
+        os.remove(obj)
+        raise RuntimeError(f"{src}: kernels using scratch memory: " + ", ".join(f"{n} ({b} B/lane)" for n, b in spilled))
 
 
 def build(force=True, verbose=False):

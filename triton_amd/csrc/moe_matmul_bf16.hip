@@ -1,7 +1,5 @@
-// Instantiates the grouped matmul kernels for one activation type: the streaming kernel for row blocks of
-// 16 (moe_matmul_stream.h), the tiled MXFP4 kernel for everything else (moe_matmul_impl.h), and the kernel for
-// unquantised weights of the same type (moe_matmul_dense.h).
-#include "moe_matmul_dense.h"
+// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for bf16 activations and routes row blocks
+// of 16 to the streaming kernel (moe_matmul_stream.h), which is compiled in moe_matmul_stream_bf16.hip.
 #include "moe_matmul_stream.h"
 
 namespace tamd {
@@ -11,14 +9,7 @@ int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStre
     block_m = 16;
     grid_m = ((a.M + 15) / 16) * a.n_experts;
   }
-  if (block_m == 16 && stream16_applicable(a)) {
-    if (a.activation == TAMD_ACT_SWIGLU) return launch_stream16<TAMD_BF16, TAMD_ACT_SWIGLU>(a, grid_m, st);
-    return launch_stream16<TAMD_BF16, TAMD_ACT_NONE>(a, grid_m, st);
-  }
+  if (block_m == 16 && stream16_applicable(a)) return stream_mm_bf16(a, grid_m, st);
   return dispatch_x16<TAMD_BF16>(a, block_m, grid_m, st);
-}
-
-int dispatch_mm_w16_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
-  return dispatch_w16<TAMD_BF16>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

@@ -1,6 +1,5 @@
-// Instantiates the grouped matmul kernels for float8_e4m3fn activations: the tiled kernel built on the scaled MFMA
-// (moe_matmul_impl.h) and, for row blocks of 16, the streaming kernel (moe_matmul_stream.h) with the rows expanded
-// to bf16 as they are loaded.
+// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for float8_e4m3fn activations (scaled MFMA) and routes row blocks
+// of 16 to the streaming kernel (moe_matmul_stream.h), which is compiled in moe_matmul_stream_fp8.hip.
 #include "moe_matmul_stream.h"
 
 namespace tamd {
@@ -10,10 +9,7 @@ int dispatch_mm_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipS
     block_m = 16;
     grid_m = ((a.M + 15) / 16) * a.n_experts;
   }
-  if (block_m == 16 && stream16_applicable(a)) {
-    if (a.activation == TAMD_ACT_SWIGLU) return launch_stream16<TAMD_BF16, TAMD_ACT_SWIGLU, true>(a, grid_m, st);
-    return launch_stream16<TAMD_BF16, TAMD_ACT_NONE, true>(a, grid_m, st);
-  }
+  if (block_m == 16 && stream16_applicable(a)) return stream_mm_fp8e4m3(a, grid_m, st);
   return dispatch_x16<TAMD_FP8_E4M3>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

@@ -223,9 +223,12 @@ constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K
 // (i, f), element j: row 32i + 8(j/4) + 4h + j%4, column t.n0 + wave*64 + c32*NF + f.
 //
 // YDT: output type fixed at compile time, or -1 to read a.y_dtype; ROWSC: per-row betas / gammas may be
-// present; FLEX: flexpoint output (expected / actual scale) may be present.  Everything that is false or
-// fixed here is a branch less per output element, and a tile has up to 160 x 256 of them.
-template <int NFR, int ACT, int YDT, bool ROWSC, bool FLEX>
+// present; FLEX: flexpoint output (expected / actual scale) may be present; MXO: MXFP8 output (a.y_mx_scale).
+// Everything that is false or fixed here is a branch less per output element, and a tile has up to
+// 160 x 256 of them.  The element loops must unroll completely (the accumulators are indexed by them and
+// would otherwise live in scratch memory), and the compiler gives up on that above a body size that one
+// variant holding every feature exceeds: hence MXO and FLEX exclude each other.
+template <int NFR, int ACT, int YDT, bool ROWSC, bool FLEX, bool MXO = false>
 TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -307,8 +310,8 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
 #pragma unroll
         for (int p = 0; p < NO; ++p) o[p] *= gamma;
       }
-      if constexpr (FLEX) {
-        if (a.y_mx_scale) {
+      if constexpr (MXO) {
+        {
           // MXFP8 output: a group is 32 consecutive output columns of a row = the outputs of one half wave (of
           // half of it when a lane holds two columns).  max |o| over the group, scale = 2^ceil(log2(max / 448)),
           // o / scale clamped to +-448; the cast below rounds to nearest even (as tamd_downcast_mxfp does).
@@ -325,13 +328,11 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
             const float q = o[p] * qs;
             o[p] = q != q ? q : __builtin_fminf(__builtin_fmaxf(q, -448.0f), 448.0f);
           }
-          // one lane per group stores the scale byte (the row may be scattered or dropped)
-          if ((c32 & (32 / NO - 1)) == 0 && r < t.rows && out_col0 < n_out) {
-            int64_t dst = t.start_m + t.off_m + r;
-            if (a.scatter_indx) dst = a.scatter_indx[dst];
-            if (dst >= 0) a.y_mx_scale[(int64_t)t.z * a.y_mx_stride_z + dst * a.y_mx_stride_m + out_col0 / 32] = (uint8_t)(sb >> 23);
-          }
+          // one lane per group leaves the scale byte behind the staged tile; the copy-out below places it
+          if ((c32 & (32 / NO - 1)) == 0) ob[NFR * 32 * OUT_COLS + r * (OUT_COLS / 32) + wave * NO + c32 * NO / 32] = (uint8_t)(sb >> 23);
         }
+      }
+      if constexpr (FLEX) {
         if (track_max && r < t.rows) {
 #pragma unroll
           for (int p = 0; p < NO; ++p)
@@ -381,6 +382,18 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
   }
   if (staged) {
     __syncthreads();
+    if constexpr (MXO) {
+      // scale bytes of the tile: OUT_COLS / 32 per row, to the row's (possibly scattered) place
+      constexpr int GPR = OUT_COLS / 32;
+      for (int id = tid; id < t.rows * GPR; id += 256) {
+        const int r = id / GPR, g = id - r * GPR;
+        const int gcol = tile_out0 + g * 32;
+        if (gcol >= n_out) continue;
+        int64_t dst = t.start_m + t.off_m + r;
+        if (a.scatter_indx) dst = a.scatter_indx[dst];
+        if (dst >= 0) a.y_mx_scale[(int64_t)t.z * a.y_mx_stride_z + dst * a.y_mx_stride_m + gcol / 32] = ob[NFR * 32 * OUT_COLS + id];
+      }
+    }
     const int epc = 16 / osz;                 // outputs per 16-byte chunk
     const int cpr = OUT_COLS / epc;           // chunks per tile row
     const int n_chunks = t.rows * cpr;
@@ -421,7 +434,9 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
 template <int NFR, int ACT, int FAST_YDT>
 TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const bool flexo = a.y_expected_scale != nullptr || a.y_actual_scale != nullptr;
-  if (a.y_dtype == FAST_YDT && !flexo) {
+  if (a.y_mx_scale) {  // always e4m3 values and no flexpoint output (checked by the entry point)
+    tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false, true>(a, t, acc, lds);
+  } else if (a.y_dtype == FAST_YDT && !flexo) {
     if (a.betas || a.gammas) tile_epilogue_t<NFR, ACT, FAST_YDT, true, false>(a, t, acc, lds);
     else tile_epilogue_t<NFR, ACT, FAST_YDT, false, false>(a, t, acc, lds);
   } else {

@@ -368,9 +368,15 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
             f[5] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 1) * mult;
             f[6] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 2) * mult;
             f[7] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 3) * mult;
-            typedef decltype(frag_t{}[0]) elem_t;
-            areg[j * 4 + u] = frag_t{(elem_t)f[0], (elem_t)f[1], (elem_t)f[2], (elem_t)f[3],
-                                     (elem_t)f[4], (elem_t)f[5], (elem_t)f[6], (elem_t)f[7]};
+            // packed by hand, two values per register: an e4m3 value times a power of two has four significant
+            // bits, so the upper half of its float32 pattern is its bf16 pattern
+            uint32_t w[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+              if constexpr (XDT == TAMD_BF16) w[p] = (f32_to_bits(f[2 * p + 1]) & 0xFFFF0000u) | (f32_to_bits(f[2 * p]) >> 16);
+              else w[p] = (f32_to_f16_bits(f[2 * p]) & 0xFFFFu) | (f32_to_f16_bits(f[2 * p + 1]) << 16);
+            }
+            areg[j * 4 + u] = __builtin_bit_cast(frag_t, make_uint4(w[0], w[1], w[2], w[3]));
           }
         }
       } else {
@@ -483,5 +489,10 @@ int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6, A8>(a, grid_m, st);
   return launch_stream16_ss<XDT, ACT, 8, A8>(a, grid_m, st);
 }
+
+// The streaming kernels of one activation type live in a translation unit of their own (moe_matmul_stream_*.hip).
+int stream_mm_bf16(const tamd_matmul_args &a, int grid_m, hipStream_t st);
+int stream_mm_f16(const tamd_matmul_args &a, int grid_m, hipStream_t st);
+int stream_mm_fp8e4m3(const tamd_matmul_args &a, int grid_m, hipStream_t st);  // fp8 rows expanded to bf16
 
 }  // namespace tamd
