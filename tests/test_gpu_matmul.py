@@ -710,3 +710,99 @@ def test_decode_row_blocks_of_16_fp8_rows(K, mx, act, device):
                      precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0) if act else None,
                      c=out_init)
     check(out, ref)
+
+
+# ---- split-K: K cut into ranges, one launch per range into float32 partial results, summed by `reduce`, activation
+# after the sum (matmul.py:180-183, 471-472, 711-737 of the reference; constraint name as in its opt_flags.py)
+@pytest.mark.parametrize("M,K,N", [(64, 2048, 512), (16, 256, 64), (33, 416, 200), (130, 2880, 520)])
+@pytest.mark.parametrize("split_k", [2, 3, 8])
+@pytest.mark.parametrize("act", [False, True])
+def test_split_k_dense(M, K, N, split_k, act, device):
+    torch.manual_seed(0)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(K, N) * 0.02
+    bias = torch.randn(N)
+    v, s, rv, rs = quantize_w(w, device)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    fa = swiglu_act(1.702, 7.0) if act else None
+    with scoped_opt_flags_constraints({"split_k": split_k}):
+        out = matmul(x.to(device), v, bias.to(device), precision_config=pc, fused_activation=fa, out_alpha=0.5)
+    ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs, out_alpha=0.5, fused_swiglu=(1.702, 7.0) if act else None)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N // 2 if act else N)
+    check(out, ref)
+
+
+@pytest.mark.parametrize("kind", ["bf16_mxfp4", "fp8_mxfp4", "mxfp8_mxfp4", "bf16_bf16"])
+def test_split_k_ragged(kind, device):
+    """Gathered rows, per-row gate weights and a bias per expert: the bias must enter once, the gate weights in
+    every range."""
+    torch.manual_seed(1)
+    E, K, N = 5, 1024, 264
+    sizes = torch.tensor([7, 0, 40, 16, 130], dtype=torch.int32)
+    M = int(sizes.sum())
+    x0 = torch.randn(M + 3, K)
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    gather = torch.randint(0, M + 3, (M, ), dtype=torch.int32)
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    kw = dict(slice_sizes=sizes, gather_indx=gather, gammas=gammas)
+    if kind == "bf16_bf16":
+        wq = w.to(torch.bfloat16)
+        xq = x0.to(torch.bfloat16)
+        pc, wdev = PrecisionConfig(), wq.to(device)
+        ref = MR.matmul_ref(xq, wq, bias, **kw)
+        xdev = xq.to(device)
+    else:
+        v, s, rv, rs = quantize_w(w, device)
+        wdev = v
+        if kind == "bf16_mxfp4":
+            xq = x0.to(torch.bfloat16)
+            xdev = xq.to(device)
+            pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+            ref = MR.matmul_ref(xq, rv, bias, b_mx_scale=rs, **kw)
+        elif kind == "fp8_mxfp4":
+            x8, x_scale = to_fp8(x0)
+            xdev = x8.to(device)
+            pc = fp8_pc(s, x_scale, device, torch.bfloat16)
+            ref = MR.matmul_ref(x8, rv, bias, a_flex_scale=x_scale, b_mx_scale=rs, **kw).to(torch.bfloat16)
+        else:
+            xdev, xs, rq, rxs = quantize_x_mxfp8(x0, device)
+            pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32)
+            ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, b_mx_scale=rs, **kw)
+    with scoped_opt_flags_constraints({"split_k": 4}):
+        out = matmul(xdev, wdev, bias.to(device), md, gather_indx=gather.to(device), precision_config=pc,
+                     gammas=gammas.to(device))
+    check(out, ref)
+
+
+def test_split_k_refuses_what_it_cannot_do(device):
+    from triton_amd.matmul import InapplicableConstraint
+    torch.manual_seed(0)
+    x = torch.randn(32, 256).to(torch.bfloat16).to(device)
+    v, s, _, _ = quantize_w(torch.randn(1, 256, 64) * 0.02, device)
+    md = make_ragged_tensor_metadata(torch.tensor([32], dtype=torch.int32, device=device), 32)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    scatter = torch.arange(32, dtype=torch.int32, device=device)
+    with scoped_opt_flags_constraints({"split_k": 2}):
+        with pytest.raises(InapplicableConstraint):
+            matmul(x, v, None, md, scatter_indx=scatter, precision_config=pc)
+
+
+@pytest.mark.parametrize("kind", ["mxfp4", "bf16"])
+def test_long_k_with_few_rows_splits_by_itself(kind, device):
+    """No constraint given: a dense problem with few rows and K >= 8192 is split without being asked."""
+    torch.manual_seed(2)
+    M, K, N = 16, 8192, 256
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(K, N) * 0.02
+    bias = torch.randn(N)
+    if kind == "mxfp4":
+        v, s, rv, rs = quantize_w(w, device)
+        out = matmul(x.to(device), v, bias.to(device), precision_config=PrecisionConfig(b_mx_scale=s, b_microblock_size=32))
+        ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs)
+    else:
+        wq = w.to(torch.bfloat16)
+        out = matmul(x.to(device), wq.to(device), bias.to(device))
+        ref = MR.matmul_ref(x, wq, bias)
+    check(out, ref)

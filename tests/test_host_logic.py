@@ -88,6 +88,9 @@ def test_opt_flags_constraints_scope_and_errors():
         with pytest.raises(OF.InapplicableConstraint):
             OF.make_opt_flags(100, 64, 64, 1, False)
     with OF.scoped_opt_flags_constraints({"split_k": 4}):
+        assert OF.make_opt_flags(100, 64, 64, 1, False).split_k == 4
+    assert OF.make_opt_flags(100, 64, 64, 1, False).split_k == 1
+    with OF.scoped_opt_flags_constraints({"split_k": 0}):
         with pytest.raises(OF.InapplicableConstraint):
             OF.make_opt_flags(100, 64, 64, 1, False)
     with OF.scoped_opt_flags_constraints({"is_persistent": True}):

@@ -299,9 +299,102 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     else:
         args.force_variant = flags.block_m if "block_m" in _opt_flags._constraints() else 0
     args.activation, args.act_alpha, args.act_limit, args.act_has_limit = act, act_alpha, act_limit, has_limit
+    split_k = flags.split_k
+    if (split_k == 1 and _opt_flags._constraints().get("split_k") is None and _opt_flags._opt_flags.get() is None
+            and not ragged and batch == 1 and M <= 256 and K >= 8192 and scatter_indx is None and not mx_out
+            and not args.y_expected_scale and not args.y_actual_scale and out.dtype.itemsize > 1
+            and args.w_mx_layout != _lib.SCALE_CDNA4):
+        # few rows and a long K: a tile's K loop is bound by the latency of its stages and there are too few
+        # tiles to hide it, so the ranges of a split run side by side (16 x 16384 x 512: 144 us -> 50 us)
+        split_k = next((s for s in (8, 4, 2) if K % (s * 128) == 0 and K // s >= 1024), 1)
+    if split_k > 1:
+        flags = OptFlags(block_m=flags.block_m, split_k=split_k)
+        _matmul_split_k(args, flags.split_k, a, wd, b.dtype == FP4, out, fused_activation, act_alpha,
+                        limit if act == _lib.ACT_SWIGLU else None, bias)
+        return finish()
     rc = _lib.lib().tamd_matmul(ctypes.byref(args), _lib.stream_ptr(a.device))
     _lib.check(rc, "matmul")
     return finish()
+
+
+def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, act_alpha, act_limit, bias):
+    """K cut into `split_k` ranges (whole multiples of 128) whose float32 partial results [split_k, B, M, N] are
+    summed afterwards (matmul.py:180-183, 471-472, 711-737 of the reference).  Every range applies the scales,
+    betas, out_alpha and gammas (all linear), only the first adds the bias (_matmul.py:523-528), and the
+    activation runs after the sum.
+
+    A plain [M, K] x [K, N] problem whose K divides evenly runs its ranges as the entries of one batched launch
+    (range s = batch entry s: activations, weights and scales advanced by s ranges, a bias that is zero for
+    s > 0), so that they share the machine; anything else gets one launch per range."""
+    from .reduce import reduce
+    from .swiglu import PrecisionConfig as SwigluPrecisionConfig, swiglu
+    if args.scatter_indx or args.y_mx_scale:
+        raise InapplicableConstraint("split_k cannot be combined with a scatter or a microscaled output")
+    if args.y_expected_scale or args.y_actual_scale or out.dtype.itemsize == 1:
+        raise InapplicableConstraint("split_k is built for 16- and 32-bit outputs without flexpoint scales")
+    if args.w_mx_layout == _lib.SCALE_CDNA4:
+        raise InapplicableConstraint("split_k needs weight scales in the strided layout")
+    K, N = args.K, args.N
+    if not w_is_fp4 and K % 64 != 0:
+        # the kernel for 16-bit weights bounds its K tail by the end of the expert's weights, which a range
+        # that starts inside them would move
+        raise InapplicableConstraint("split_k with 16-bit weights needs K to be a multiple of 64")
+    chunk = -(-(-(-K // split_k)) // 128) * 128
+    n_split = -(-K // chunk)
+    batch, rows = out.shape[0], out.shape[1]
+    scratch = torch.empty((n_split, batch, rows, N), dtype=torch.float32, device=out.device)
+    w_esz = 1 if w_is_fp4 else wd.element_size()
+    one_launch = args.n_experts == 1 and not args.block_schedule and batch == 1 and K % chunk == 0
+    if one_launch:
+        kq = chunk // 2 if w_is_fp4 else chunk
+        part = type(args).from_buffer_copy(args)
+        part.K, part.n_experts = chunk, n_split
+        part.x_stride_z = chunk
+        part.w_stride_e = kq * args.w_stride_k
+        if args.w_mx_scale:
+            part.w_mx_stride_e = (chunk // MXFP_BLOCK_SIZE) * args.w_mx_stride_k
+        if args.x_mx_scale:
+            part.x_mx_stride_z = chunk // MXFP_BLOCK_SIZE
+        if bias is not None:
+            bias_s = torch.zeros((n_split, N), dtype=torch.float32, device=out.device)
+            bias_s[0] = bias.reshape(-1)
+            part.bias, part.bias_dtype, part.bias_stride_e = bias_s.data_ptr(), _lib.F32, N
+        part.activation = _lib.ACT_NONE
+        part.y, part.y_dtype = scratch.data_ptr(), _lib.F32
+        part.y_stride_m, part.y_stride_z = scratch.stride(2), scratch.stride(0)
+        part.force_variant = 0
+        rc = _lib.lib().tamd_matmul(ctypes.byref(part), _lib.stream_ptr(out.device))
+        _lib.check(rc, "matmul (split_k ranges as a batch)")
+    for s in range(0 if one_launch else n_split):
+        k0 = s * chunk
+        part = type(args).from_buffer_copy(args)
+        part.K = min(chunk, K - k0)
+        part.x = args.x + k0 * a.element_size()
+        part.w = args.w + (k0 // 2 if w_is_fp4 else k0) * args.w_stride_k * w_esz
+        if args.w_mx_scale:
+            part.w_mx_scale = args.w_mx_scale + (k0 // MXFP_BLOCK_SIZE) * args.w_mx_stride_k
+        if args.x_mx_scale:
+            part.x_mx_scale = args.x_mx_scale + k0 // MXFP_BLOCK_SIZE
+        if s > 0:
+            part.bias = None
+        part.activation = _lib.ACT_NONE
+        part.y, part.y_dtype = scratch[s].data_ptr(), _lib.F32
+        part.y_stride_m, part.y_stride_z = scratch.stride(2), scratch.stride(1)
+        rc = _lib.lib().tamd_matmul(ctypes.byref(part), _lib.stream_ptr(out.device))
+        _lib.check(rc, "matmul (split_k range)")
+    parts = scratch.view(n_split, batch * rows, N)
+    direct = out.is_contiguous() and fused_activation.specs.name == "dflt"
+    if direct:
+        reduce(parts, dim=0, y=out.view(batch * rows, N), y_dtype=out.dtype)
+        return
+    total, _ = reduce(parts, dim=0, y_dtype=torch.float32)
+    if fused_activation.specs.name == "swiglu":
+        total = swiglu(total, act_alpha, SwigluPrecisionConfig(act_limit))
+    if out.is_contiguous():
+        # float32 -> output type with the library's own kernel: a sum over an axis of length one
+        reduce(total[None], dim=0, y=out.view(batch * rows, -1), y_dtype=out.dtype)
+    else:
+        out.copy_(total.view(out.shape))
 
 
 matmul_ogs = matmul

@@ -84,8 +84,10 @@ def make_opt_flags(m: int, n: int, k: int, n_slices: int, ragged: bool,
     for key in ("is_persistent", ):
         if c.get(key):
             raise InapplicableConstraint("there is no persistent kernel on gfx950")
-    if c.get("split_k", 1) not in (1, None):
-        raise InapplicableConstraint("split_k > 1 is not built")
+    split_k = c.get("split_k")
+    split_k = 1 if split_k is None else int(split_k)
+    if split_k < 1:
+        raise InapplicableConstraint("split_k must be positive")
     rows = m
     if ragged:
         rows = expected_slice_size if expected_slice_size is not None else max(1, m // max(1, n_slices))
@@ -94,4 +96,4 @@ def make_opt_flags(m: int, n: int, k: int, n_slices: int, ragged: bool,
         block_m = int(c["block_m"])
         if block_m not in BLOCK_M_CHOICES:
             raise InapplicableConstraint(f"block_m must be one of {BLOCK_M_CHOICES}")
-    return OptFlags(block_m=block_m)
+    return OptFlags(block_m=block_m, split_k=split_k)
