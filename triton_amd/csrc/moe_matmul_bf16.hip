@@ -1,5 +1,6 @@
-// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for bf16 activations and routes row blocks
-// of 16 to the streaming kernel (moe_matmul_stream.h), which is compiled in moe_matmul_stream_bf16.hip.
+// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for bf16 activations with the plain epilogue
+// (the SwiGLU ones are compiled in moe_matmul_bf16_swiglu.hip) and routes row blocks of 16 to the streaming kernel
+// (moe_matmul_stream.h), which is compiled in moe_matmul_stream_bf16.hip.
 #include "moe_matmul_stream.h"
 
 namespace tamd {
@@ -10,6 +11,7 @@ int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStre
     grid_m = ((a.M + 15) / 16) * a.n_experts;
   }
   if (block_m == 16 && stream16_applicable(a)) return stream_mm_bf16(a, grid_m, st);
-  return dispatch_x16<TAMD_BF16>(a, block_m, grid_m, st);
+  if (a.activation == TAMD_ACT_SWIGLU) return tiled_mm_swiglu_bf16(a, block_m, grid_m, st);
+  return dispatch_x16_act<TAMD_BF16, TAMD_ACT_NONE>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

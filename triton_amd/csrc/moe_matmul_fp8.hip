@@ -1,5 +1,6 @@
-// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for float8_e4m3fn activations (scaled MFMA) and routes row blocks
-// of 16 to the streaming kernel (moe_matmul_stream.h), which is compiled in moe_matmul_stream_fp8.hip.
+// Instantiates the tiled MXFP4 grouped matmul kernels (moe_matmul_impl.h) for float8_e4m3fn activations (scaled MFMA) with the plain epilogue
+// (the SwiGLU ones are compiled in moe_matmul_fp8_swiglu.hip) and routes row blocks of 16 to the streaming kernel
+// (moe_matmul_stream.h), which is compiled in moe_matmul_stream_fp8.hip.
 #include "moe_matmul_stream.h"
 
 namespace tamd {
@@ -10,6 +11,7 @@ int dispatch_mm_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipS
     grid_m = ((a.M + 15) / 16) * a.n_experts;
   }
   if (block_m == 16 && stream16_applicable(a)) return stream_mm_fp8e4m3(a, grid_m, st);
-  return dispatch_x16<TAMD_FP8_E4M3>(a, block_m, grid_m, st);
+  if (a.activation == TAMD_ACT_SWIGLU) return tiled_mm_swiglu_fp8e4m3(a, block_m, grid_m, st);
+  return dispatch_x16_act<TAMD_FP8_E4M3, TAMD_ACT_NONE>(a, block_m, grid_m, st);
 }
 }  // namespace tamd

@@ -808,12 +808,6 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   return launch_status();
 }
 
-template <int XDT, int BM>
-int launch_x16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  if (a.activation == TAMD_ACT_SWIGLU) return launch_x16_act<XDT, BM, TAMD_ACT_SWIGLU>(a, grid_m, st);
-  return launch_x16_act<XDT, BM, TAMD_ACT_NONE>(a, grid_m, st);
-}
-
 // Row block size of a dense / batched problem (block_m == 0 on entry of a dispatcher): the largest block whose
 // tiles still give every CU one, because a tile's K loop is bound by the latency of its stages, not by its
 // rows -- 256 x 2048 x 4096 runs 55 us as 2 x 16 tiles of 128 rows and 27 us as 8 x 16 tiles of 32.
@@ -830,16 +824,22 @@ inline void dense_grid(const tamd_matmul_args &a, int &block_m, int &grid_m) {
   grid_m = ((a.M + block_m - 1) / block_m) * a.n_experts;
 }
 
-template <int XDT>
-int dispatch_x16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+// The tiled kernels of one activation type and one epilogue activation.  The two activations are compiled in
+// translation units of their own (moe_matmul_<type>.hip: none, moe_matmul_<type>_swiglu.hip: SwiGLU), which
+// is all that separates them: each unit holds 16 kernels of up to 20 unrolled epilogues.
+template <int XDT, int ACT>
+int dispatch_x16_act(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
   dense_grid(a, block_m, grid_m);
   switch (block_m) {
-    case 16: return launch_x16<XDT, 16>(a, grid_m, st);
-    case 32: return launch_x16<XDT, 32>(a, grid_m, st);
-    case 64: return launch_x16<XDT, 64>(a, grid_m, st);
-    case 128: return launch_x16<XDT, 128>(a, grid_m, st);
+    case 16: return launch_x16_act<XDT, 16, ACT>(a, grid_m, st);
+    case 32: return launch_x16_act<XDT, 32, ACT>(a, grid_m, st);
+    case 64: return launch_x16_act<XDT, 64, ACT>(a, grid_m, st);
+    case 128: return launch_x16_act<XDT, 128, ACT>(a, grid_m, st);
     default: return TAMD_E_UNSUPPORTED;
   }
 }
+int tiled_mm_swiglu_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int tiled_mm_swiglu_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int tiled_mm_swiglu_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 
 }  // namespace tamd
