@@ -161,7 +161,7 @@ int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, i
 typedef struct tamd_matmul_args {
   /* activations: [M_x, K], unit stride along K */
   const void *x;
-  int x_dtype; /* TAMD_BF16 / TAMD_F16 / TAMD_FP8_E4M3 */
+  int x_dtype; /* TAMD_BF16 / TAMD_F16 / TAMD_FP8_E4M3 / TAMD_FP8_E5M2 */
   int64_t x_stride_m;
   const float *x_scale; /* per-tensor flex scale (device scalar) or NULL */
   /* weights: n_experts x [K, N]; MXFP4: packed bytes, K/2 bytes contiguous per column.  TAMD_BF16 / TAMD_F16

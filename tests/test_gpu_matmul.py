@@ -158,42 +158,45 @@ def test_empty(device):
 # ---------------------------------------------------------------------------- fp8 activations (scaled MFMA)
 
 
-def to_fp8(x0):
-    """Per-tensor flex quantisation as in BASELINE config 5: s = amax / 448, x = (x0 / s) -> e4m3."""
+def to_fp8(x0, fp8=torch.float8_e4m3fn):
+    """Per-tensor flex quantisation as in BASELINE config 5: s = amax / 448, x = (x0 / s) -> e4m3 (or e5m2: the
+    activation type of most fp8 cases of the reference, tests/test_matmul.py:150-196)."""
     s = x0.abs().max() / 448.0
-    return (x0 / s).to(torch.float8_e4m3fn), s.reshape(1).float()
+    return (x0 / s).to(fp8), s.reshape(1).float()
 
 
-def fp8_pc(s_w, x_scale, device, out_dtype):
-    flex = FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale.to(device)))
+def fp8_pc(s_w, x_scale, device, out_dtype, fp8=torch.float8_e4m3fn):
+    flex = FlexCtx(lhs_data=InFlexData(dtype=fp8, scale=x_scale.to(device)))
     return PrecisionConfig(b_mx_scale=s_w, b_microblock_size=32, flex_ctx=flex, out_dtype=out_dtype)
 
 
 @pytest.mark.parametrize("M,K,N", [(256, 2048, 512), (16, 64, 64), (33, 96, 200), (130, 192, 520), (1, 32, 16),
                                    (128, 2880, 256)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_fp8_dense(M, K, N, out_dtype, device):
+@pytest.mark.parametrize("fp8", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_fp8_dense(M, K, N, out_dtype, fp8, device):
     torch.manual_seed(0)
-    x8, xs = to_fp8(torch.randn(M, K))
+    x8, xs = to_fp8(torch.randn(M, K), fp8)
     w = torch.randn(K, N) * 0.02
     bias = torch.randn(N) * 0.1
     v, s, rv, rs = quantize_w(w, device)
-    out = matmul(x8.to(device), v, bias.to(device), precision_config=fp8_pc(s, xs, device, out_dtype))
+    out = matmul(x8.to(device), v, bias.to(device), precision_config=fp8_pc(s, xs, device, out_dtype, fp8))
     ref = MR.matmul_ref(x8, rv, bias, b_mx_scale=rs, a_flex_scale=xs)
     assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
     check(out, ref.to(out_dtype))
 
 
-def test_fp8_one_hot_rows_are_exact(device):
+@pytest.mark.parametrize("fp8", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_fp8_one_hot_rows_are_exact(fp8, device):
     """x = one-hot rows (1.0 is exact in e4m3): the scaled MFMA must return the dequantised weight rows bit for
     bit, which pins the K order of both operands and the scale-byte selection."""
     torch.manual_seed(1)
     K, N = 256, 256
     w = torch.randn(K, N)
     v, s, rv, rs = quantize_w(w, device)
-    x8 = torch.eye(K)[:160].to(torch.float8_e4m3fn)
+    x8 = torch.eye(K)[:160].to(fp8)
     one = torch.ones(1)
-    out = matmul(x8.to(device), v, None, precision_config=fp8_pc(s, one, device, torch.float32))
+    out = matmul(x8.to(device), v, None, precision_config=fp8_pc(s, one, device, torch.float32, fp8))
     from oracle.mxfp_ref import upcast_from_mxfp_ref
     deq = upcast_from_mxfp_ref(rv, rs, torch.float32, axis=0)
     assert torch.equal(out.cpu(), deq[:160])
@@ -202,11 +205,12 @@ def test_fp8_one_hot_rows_are_exact(device):
 @pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128])
 @pytest.mark.parametrize("do_gather,do_scatter,do_gamma,act", [(False, False, False, False), (True, False, False, True),
                                                                 (False, True, True, False)])
-def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, device):
+@pytest.mark.parametrize("fp8", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, fp8, device):
     torch.manual_seed(0)
     E, K, N, M = 9, 320, 392, 700
     sizes = torch.tensor([0, 5, 130, 16, 1, 257, 64, 200, 27], dtype=torch.int32)
-    x8, xs = to_fp8(torch.randn(M, K))
+    x8, xs = to_fp8(torch.randn(M, K), fp8)
     w = torch.randn(E, K, N) * 0.05
     bias = torch.randn(E, N)
     v, s, rv, rs = quantize_w(w, device)
@@ -221,7 +225,7 @@ def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, device):
     out_init = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=device)
     with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
         out = matmul(dev(x8), v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter),
-                     precision_config=fp8_pc(s, xs, device, torch.bfloat16), gammas=dev(gammas), fused_activation=fa,
+                     precision_config=fp8_pc(s, xs, device, torch.bfloat16, fp8), gammas=dev(gammas), fused_activation=fa,
                      c=out_init)
     ref = MR.matmul_ref(x8, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs,
                         a_flex_scale=xs, gammas=gammas, fused_swiglu=(1.702, 7.0) if act else None)
@@ -675,10 +679,10 @@ def test_mxfp8_output_ragged_then_mxfp8_input(block_m, device):
 
 
 @pytest.mark.parametrize("K", [64, 1024, 2880, 4096])
-@pytest.mark.parametrize("mx", [False, True])
+@pytest.mark.parametrize("mx", [False, True, "e5m2"])
 @pytest.mark.parametrize("act", [False, True])
 def test_decode_row_blocks_of_16_fp8_rows(K, mx, act, device):
-    """The streaming kernel with float8_e4m3fn rows (per-tensor flex scale, or MXFP8 block scales), expanded to bf16
+    """The streaming kernel with fp8 rows (e4m3 with a per-tensor flex scale or MXFP8 block scales; e5m2 with a flex scale), expanded to bf16
     as a row block is loaded; gather, scatter with dropped rows, gate weights."""
     torch.manual_seed(K)
     E, N = 7, 608
@@ -695,14 +699,15 @@ def test_decode_row_blocks_of_16_fp8_rows(K, mx, act, device):
     md = make_ragged_tensor_metadata(sizes.to(device), M)
     kw = dict(slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs, gammas=gammas,
               fused_swiglu=(1.702, 7.0) if act else None)
-    if mx:
+    if mx is True:
         xq, xs, rq, rxs = quantize_x_mxfp8(x0, device)
         pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32)
         ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, **kw)
     else:
-        x8, x_scale = to_fp8(x0)
+        fp8 = torch.float8_e5m2 if mx == "e5m2" else torch.float8_e4m3fn
+        x8, x_scale = to_fp8(x0, fp8)
         xq = x8.to(device)
-        pc = fp8_pc(s, x_scale, device, torch.bfloat16)
+        pc = fp8_pc(s, x_scale, device, torch.bfloat16, fp8)
         ref = MR.matmul_ref(x8, rv, bias, a_flex_scale=x_scale, **kw).to(torch.bfloat16)
     out_init = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=device)
     with scoped_opt_flags_constraints({"block_m": 16}):

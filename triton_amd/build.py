@@ -13,6 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtriton_amd.so")
 SOURCES = ["api.cpp", "mxfp.hip", "routing.hip", "elementwise.hip", "moe_matmul.hip", "moe_matmul_bf16.hip", "moe_matmul_f16.hip",
            "moe_matmul_fp8.hip", "moe_matmul_bf16_swiglu.hip", "moe_matmul_f16_swiglu.hip", "moe_matmul_fp8_swiglu.hip",
+           "moe_matmul_fp8e5m2.hip", "moe_matmul_fp8e5m2_swiglu.hip", "moe_matmul_stream_fp8e5m2.hip",
            "moe_matmul_stream_bf16.hip", "moe_matmul_stream_f16.hip", "moe_matmul_stream_fp8.hip",
            "moe_matmul_w16_bf16.hip", "moe_matmul_w16_f16.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -7,6 +7,7 @@ namespace tamd {
 int dispatch_mm_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int dispatch_mm_fp8e5m2(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_w16_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int dispatch_mm_w16_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 }  // namespace tamd
@@ -32,7 +33,7 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
   if (ragged && (!a.slice_sizes || !a.slice_offs || a.grid_m < 0)) return TAMD_E_INVALID;
   hipStream_t st = (hipStream_t)stream;
 
-  const bool x8 = a.x_dtype == TAMD_FP8_E4M3;
+  const bool x8 = a.x_dtype == TAMD_FP8_E4M3 || a.x_dtype == TAMD_FP8_E5M2;
   if (a.w_dtype == TAMD_MXFP4 && (a.x_dtype == TAMD_BF16 || a.x_dtype == TAMD_F16 || x8)) {
     const int esz = x8 ? 1 : 2;
     if (!a.w_mx_scale) return TAMD_E_INVALID;
@@ -65,6 +66,7 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     }
     if (a.x_dtype == TAMD_BF16) return dispatch_mm_bf16(a, block_m, grid_m, st);
     if (a.x_dtype == TAMD_F16) return dispatch_mm_f16(a, block_m, grid_m, st);
+    if (a.x_dtype == TAMD_FP8_E5M2) return dispatch_mm_fp8e5m2(a, block_m, grid_m, st);
     return dispatch_mm_fp8e4m3(a, block_m, grid_m, st);
   }
   if ((a.x_dtype == TAMD_BF16 || a.x_dtype == TAMD_F16) && a.w_dtype == a.x_dtype) {

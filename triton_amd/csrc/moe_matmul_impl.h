@@ -841,5 +841,6 @@ int dispatch_x16_act(const tamd_matmul_args &a, int block_m, int grid_m, hipStre
 int tiled_mm_swiglu_bf16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int tiled_mm_swiglu_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 int tiled_mm_swiglu_fp8e4m3(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
+int tiled_mm_swiglu_fp8e5m2(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st);
 
 }  // namespace tamd

@@ -62,6 +62,13 @@ TAMD_DEVICE void dma16_at(v4i_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t
                  : "memory");
 }
 
+// byte SEL of a dword as float32 (the selector of the conversion is an immediate)
+template <int A8, int SEL>
+TAMD_DEVICE float fp8_byte(uint32_t word) {
+  if constexpr (A8 == 2) return __builtin_amdgcn_cvt_f32_bf8((int)word, SEL);
+  else return __builtin_amdgcn_cvt_f32_fp8((int)word, SEL);
+}
+
 template <int SS, int RING_>
 struct StreamShape {
   static constexpr int CODE_BYTES = 4 * SS * 1024;  // image of 16 columns' codes, padded to whole 1 KB copies
@@ -82,9 +89,10 @@ struct StreamShape {
 // issue and await the copies, waves 6-7 finish and store the previous unit.  A wave that issues copies
 // stalls whenever the memory pipeline is full; with nothing else to do it refills the pipeline the
 // moment there is room, and the stalls never delay MFMA work or stores.
-// A8: the activations are stored as float8_e4m3fn (optionally with e8m0 block scales per 32 K) and are expanded to
+// A8 (1: float8_e4m3fn, 2: float8_e5m2; 0: rows of XDT): the activations are stored as fp8 (optionally with e8m0 block
+// scales per 32 K) and are expanded to
 // XDT when a row block's slice is loaded into registers -- exact, so the K loop is the same as for 16-bit rows.
-template <int XDT, int ACT, int SS, int RING, bool A8>
+template <int XDT, int ACT, int SS, int RING, int A8>
 __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
@@ -360,15 +368,15 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
             uint2 v = make_uint2(0, 0);
             if (live) v = *(const uint2 *)(xr + 32 * kg + 8 * u);
             float f[8];
-            f[0] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 0) * mult;
-            f[1] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 1) * mult;
-            f[2] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 2) * mult;
-            f[3] = __builtin_amdgcn_cvt_f32_fp8((int)v.x, 3) * mult;
-            f[4] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 0) * mult;
-            f[5] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 1) * mult;
-            f[6] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 2) * mult;
-            f[7] = __builtin_amdgcn_cvt_f32_fp8((int)v.y, 3) * mult;
-            // packed by hand, two values per register: an e4m3 value times a power of two has four significant
+            f[0] = fp8_byte<A8, 0>(v.x) * mult;
+            f[1] = fp8_byte<A8, 1>(v.x) * mult;
+            f[2] = fp8_byte<A8, 2>(v.x) * mult;
+            f[3] = fp8_byte<A8, 3>(v.x) * mult;
+            f[4] = fp8_byte<A8, 0>(v.y) * mult;
+            f[5] = fp8_byte<A8, 1>(v.y) * mult;
+            f[6] = fp8_byte<A8, 2>(v.y) * mult;
+            f[7] = fp8_byte<A8, 3>(v.y) * mult;
+            // packed by hand, two values per register: an fp8 value times a power of two has at most four significant
             // bits, so the upper half of its float32 pattern is its bf16 pattern
             uint32_t w[4];
 #pragma unroll
@@ -462,7 +470,7 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   return true;
 }
 
-template <int XDT, int ACT, int SS, bool A8>
+template <int XDT, int ACT, int SS, int A8>
 int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + (SS + 1) / 2 * 1024 + 256);
   constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
@@ -481,7 +489,7 @@ int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   return launch_status();
 }
 
-template <int XDT, int ACT, bool A8 = false>
+template <int XDT, int ACT, int A8 = 0>
 int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int ss = (a.K / 32 + 15) / 16;  // super steps per wave
   if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2, A8>(a, grid_m, st);
@@ -494,5 +502,6 @@ int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
 int stream_mm_bf16(const tamd_matmul_args &a, int grid_m, hipStream_t st);
 int stream_mm_f16(const tamd_matmul_args &a, int grid_m, hipStream_t st);
 int stream_mm_fp8e4m3(const tamd_matmul_args &a, int grid_m, hipStream_t st);  // fp8 rows expanded to bf16
+int stream_mm_fp8e5m2(const tamd_matmul_args &a, int grid_m, hipStream_t st);
 
 }  // namespace tamd

@@ -83,7 +83,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     """
     Y[dst(r), :] = act((X[src(r), :] @ W[e]) + bias[e] * betas[r]) * gammas[r]   for the rows r of every slice e
 
-    a: [M, K] activations (bf16 / fp16, or float8_e4m3fn with flex_ctx.lhs_data.scale), or [B, M, K] batched.
+    a: [M, K] activations (bf16 / fp16, or float8_e4m3fn / float8_e5m2 with flex_ctx.lhs_data.scale), or [B, M, K] batched.
     b: [E, K, N] weights; MXFP4 weights are uint8 with two codes per byte along K
        (storage [E, K/2, N] with unit stride along K) and precision_config.b_mx_scale
        holds their e8m0 scales [E, K/32, N].
