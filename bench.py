@@ -264,8 +264,8 @@ def run_fc2(args, cfg):
     n_chk = 2048
     combine_ok = bool(torch.equal(z[:n_chk].cpu(), MR.reduce_ref(y.view(T, k, N)[:n_chk].cpu(), 1)))
     cpu, gemm_ok = None, None
-    if args.cpu_experts > 0:
-        n_e = min(args.cpu_experts, E)
+    if args.cpu_experts != 0:
+        n_e = min(args.cpu_experts, E) if args.cpu_experts > 0 else max(1, min(E, int(6e11 / (2.0 * rows / E * K * N))))
         y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x8.cpu(), vals, scales, bias_cpu, ref, n_e, K, N, False,
                                                         fc2=(x_scale.cpu(), gam_ref))
         got = y.cpu()[ref["scatter_indx"][:n_rows].long()]
@@ -293,7 +293,8 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="fc1_prefill", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-experts", type=int, default=8, help="experts in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-experts", type=int, default=-1,
+                    help="experts in the CPU baseline sample (0 = skip; default: about 0.6 TFLOP of oracle work, 10-15 s)")
     ap.add_argument("--block-m", type=int, default=0)
     ap.add_argument("--scale-layout", default="strided", choices=["strided", "cdna4"],
                     help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
@@ -403,8 +404,8 @@ def main():
                       and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]))
     cpu = None
     gemm_ok = None
-    if args.cpu_experts > 0:
-        n_e = min(args.cpu_experts, E)
+    if args.cpu_experts != 0:
+        n_e = min(args.cpu_experts, E) if args.cpu_experts > 0 else max(1, min(E, int(6e11 / (2.0 * rows / E * K * N))))
         x_ref = x_cpu
         if mx8:  # the oracle sees the same quantised activations, dequantised (exactly) to bf16
             from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
