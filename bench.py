@@ -397,6 +397,12 @@ def main():
     roof["algorithmic_flops"] = flops
     roof["frac_of_mxfp4_peak"] = round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4)
     roof["hbm_gbs"] = round(gbs_kernel, 1)
+    if rows > 16 * E:
+        # the tiled kernel computes whole 32-row MFMA fragments: rows of the ragged experts rounded up to 32 are what
+        # the matrix cores actually run (the share that is padding is the price of the ragged row counts)
+        issued_rows = int(((col_sum + 31) // 32 * 32).sum())
+        roof["mfma_rows_issued"] = issued_rows
+        roof["mfma_issue_tflops"] = round(2.0 * issued_rows * K * N / (kernel_ms * 1e-3) / 1e12, 1)
 
     # parity of this very run against the oracle, and the CPU baseline, on a bounded sample
     ref = RR.routing_ref(logits_cpu, k)
