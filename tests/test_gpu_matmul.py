@@ -811,3 +811,31 @@ def test_long_k_with_few_rows_splits_by_itself(kind, device):
         out = matmul(x.to(device), wq.to(device), bias.to(device))
         ref = MR.matmul_ref(x, wq, bias)
     check(out, ref)
+
+
+@pytest.mark.parametrize("fp8", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("ragged", [False, True])
+def test_mxfp8_weights(fp8, ragged, device):
+    """bfloat16 x MXFP8 weights (tests/test_matmul.py:177-178 of the reference): the weights are dequantised to
+    bfloat16 by the upcast kernel and multiplied by the kernel for unquantised weights."""
+    from oracle.mxfp_ref import downcast_to_mxfp_ref as dref
+    torch.manual_seed(3)
+    E, K, N = (4, 320, 264) if ragged else (1, 416, 200)
+    sizes = torch.tensor([40, 0, 130, 9], dtype=torch.int32)
+    M = int(sizes.sum()) if ragged else 70
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s = downcast_to_mxfp(w.to(device), fp8, axis=-2)
+    rv, rs = dref(w, fp8, axis=-2)
+    assert torch.equal(v.cpu().view(torch.uint8), rv.view(torch.uint8)) and torch.equal(s.cpu(), rs)
+    pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    if ragged:
+        md = make_ragged_tensor_metadata(sizes.to(device), M)
+        out = matmul(x.to(device), v, bias.to(device), md, precision_config=pc)
+        ref = MR.matmul_ref(x, rv, bias, slice_sizes=sizes, b_mx_scale=rs)
+    else:
+        pc = PrecisionConfig(b_mx_scale=s[0], b_microblock_size=32)
+        out = matmul(x.to(device), v[0], bias[0].to(device), precision_config=pc)
+        ref = MR.matmul_ref(x, rv[0], bias[0], b_mx_scale=rs[0])
+    check(out, ref)

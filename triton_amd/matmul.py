@@ -151,6 +151,17 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         assert b_scale.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.dtype}"
     if isinstance(a, Tensor):
         a = a.storage.data
+    if b_scale is not None and b.dtype != FP4:
+        # MXFP8 weights: dequantised to bfloat16 by the library's upcast kernel, as the reference's torch path does
+        # (matmul.py:788-794), and multiplied by the kernel for unquantised weights
+        w8 = b.storage.data
+        if w8.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2) or b_scale_cdna4:
+            raise NotImplementedError("microscaled weights are built as MXFP4, or MXFP8 with scales in the strided layout")
+        if a.dtype != torch.bfloat16 or a_mx_scale is not None:
+            raise NotImplementedError("MXFP8 weights are built for bfloat16 activations")
+        from .numerics_details.mxfp import upcast_from_mxfp
+        b = wrap_torch_tensor(upcast_from_mxfp(w8, b_scale, torch.bfloat16, axis=-2))
+        b_scale = None
     a = flex.lhs_data.reinterpret(a)
     w = flex.rhs_data.reinterpret(b.storage.data)
     _lib.require_gpu(a, "a")
