@@ -301,8 +301,8 @@ def main():
                     "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout()))")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (experts would shard across GPUs, "
-              "see DESIGN.md)", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (with more GPUs the experts "
+              "would be sharded across them, one exchange of rows before and after the two matmuls)", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
