@@ -41,10 +41,12 @@ def test_alias():
     assert matmul_ogs is matmul
 
 
-@pytest.mark.parametrize("M,K,N", [(256, 2048, 4096), (16, 64, 64), (33, 96, 200), (130, 192, 520), (1, 32, 16)])
+@pytest.mark.parametrize("M,K,N", [(256, 2048, 4096), (16, 64, 64), (33, 96, 200), (130, 192, 520), (1, 32, 16),
+                                   (15, 96, 66), (40, 160, 322)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_dense(M, K, N, dtype, device):
-    """(256, 2048, 4096) is BASELINE config 1."""
+    """(256, 2048, 4096) is BASELINE config 1; (15, 96, 66) and (40, 160, 322) have scale images whose size is not a
+    multiple of four bytes (the last columns' scales sit in a partial dword)."""
     torch.manual_seed(0)
     x = torch.randn(M, K).to(dtype)
     w = torch.randn(K, N) * 0.02

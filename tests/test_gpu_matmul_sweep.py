@@ -1,0 +1,109 @@
+"""GPU parity: a seeded sweep over combinations the hand-written cases of test_gpu_matmul.py do not enumerate --
+activation type x row-block size x weight-scale layout x gather / scatter / betas / gammas / bias type x output type x
+SwiGLU, on ragged problems with random (often empty or tiny) slices and odd sizes.  Every case goes through the C
+ABI and is compared with the CPU oracle (rtol = atol = 1e-2 on the scale of the outputs, see `check`)."""
+import random
+
+import pytest
+import torch
+
+from oracle import matmul_ref as MR
+from oracle.mxfp_ref import downcast_to_mxfp_ref
+from triton_amd.matmul import FlexCtx, FnSpecs, FusedActivation, InFlexData, PrecisionConfig, matmul
+from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
+from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+from triton_amd.swiglu import swiglu_fn
+from triton_amd.tensor import convert_layout, make_ragged_tensor_metadata, wrap_torch_tensor
+from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
+from triton_amd.testing import assert_close
+
+pytestmark = pytest.mark.gpu
+
+KINDS = ["bf16", "f16", "e4m3", "e5m2", "mxfp8"]
+
+
+def make_case(seed):
+    rng = random.Random(seed)
+    c = dict(seed=seed)
+    c["kind"] = KINDS[seed % len(KINDS)]
+    c["E"] = rng.choice([1, 2, 5, 9])
+    c["K"] = 32 * rng.choice([1, 2, 3, 5, 10, 13, 32, 45])
+    c["N"] = 2 * rng.choice([8, 16, 33, 100, 128, 131, 264, 300])
+    c["sizes"] = [rng.choice([0, 1, 2, 15, 16, 17, 31, 33, 64, 100, 129, 161, 260]) for _ in range(c["E"])]
+    if sum(c["sizes"]) == 0:
+        c["sizes"][0] = 7
+    c["block_m"] = rng.choice([None, 16, 32, 64, 128])
+    c["cdna4"] = rng.random() < 0.4
+    c["gather"], c["scatter"] = rng.random() < 0.5, rng.random() < 0.5
+    c["betas"], c["gammas"] = rng.random() < 0.3, rng.random() < 0.5
+    c["bias"] = rng.choice([None, torch.float32, torch.bfloat16, torch.float16])
+    c["act"] = rng.random() < 0.5
+    c["out"] = rng.choice([None, torch.float32]) if c["kind"] in ("bf16", "f16") else rng.choice([torch.bfloat16, torch.float32])
+    return c
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_sweep(seed, device):
+    c = make_case(seed)
+    print("case", c, flush=True)
+    torch.manual_seed(seed)
+    E, K, N = c["E"], c["K"], c["N"]
+    sizes = torch.tensor(c["sizes"], dtype=torch.int32)
+    M = int(sizes.sum())
+    n_src = M + 3
+    x0 = torch.randn(n_src, K)
+    w = torch.randn(E, K, N) * 0.05
+    v, s = downcast_to_mxfp(w.to(device), torch.uint8, axis=-2)
+    rv, rs = downcast_to_mxfp_ref(w, torch.uint8, axis=-2)
+    assert torch.equal(v.cpu(), rv) and torch.equal(s.cpu(), rs)
+    sc = convert_layout(wrap_torch_tensor(s), CDNA4MXScaleLayout()) if c["cdna4"] else s
+    bias = None if c["bias"] is None else torch.randn(E, N).to(c["bias"])
+    gather = torch.randint(0, n_src, (M, ), dtype=torch.int32) if c["gather"] else None
+    scatter = None
+    if c["scatter"]:
+        scatter = torch.randperm(M, dtype=torch.int32)
+        scatter[::5] = -1
+    betas = 2.0**torch.randint(-2, 2, (M, )).float() if c["betas"] else None
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float() if c["gammas"] else None
+    kw = dict(slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, b_mx_scale=rs, betas=betas, gammas=gammas,
+              fused_swiglu=(1.702, 7.0) if c["act"] else None)
+    kind = c["kind"]
+    if kind in ("bf16", "f16"):
+        dt = torch.bfloat16 if kind == "bf16" else torch.float16
+        xq = x0.to(dt)
+        xdev = xq.to(device)
+        pc = PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=c["out"])
+        ref = MR.matmul_ref(xq if gather is not None else xq[:M], rv, bias, **kw)
+        if gather is None:
+            xdev = xdev[:M]
+        out_dtype = c["out"] or dt
+    elif kind in ("e4m3", "e5m2"):
+        fp8 = torch.float8_e4m3fn if kind == "e4m3" else torch.float8_e5m2
+        x_scale = (x0.abs().max() / 448.0).reshape(1).float()
+        xq = (x0 / x_scale).to(fp8)
+        xdev = xq.to(device) if gather is not None else xq[:M].to(device)
+        pc = PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=c["out"],
+                             flex_ctx=FlexCtx(lhs_data=InFlexData(dtype=fp8, scale=x_scale.to(device))))
+        ref = MR.matmul_ref(xq if gather is not None else xq[:M], rv, bias, a_flex_scale=x_scale, **kw)
+        out_dtype = c["out"]
+    else:
+        x0 = x0 * torch.exp(torch.randn(n_src, K // 32).repeat_interleave(32, dim=1))
+        xv, xs = downcast_to_mxfp(x0.to(device), torch.float8_e4m3fn, axis=-1)
+        rq, rxs = downcast_to_mxfp_ref(x0, torch.float8_e4m3fn, axis=-1)
+        assert torch.equal(xv.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs.cpu(), rxs)
+        if gather is None:
+            xv, xs, rq, rxs = xv[:M], xs[:M], rq[:M], rxs[:M]
+        xdev = xv
+        pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=sc, b_microblock_size=32, out_dtype=c["out"])
+        ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, **kw)
+        out_dtype = c["out"]
+    dev = lambda t: None if t is None else t.to(device)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if c["act"] else None
+    out_init = torch.zeros((M, N // 2 if c["act"] else N), dtype=out_dtype, device=device)
+    with scoped_opt_flags_constraints({} if c["block_m"] is None else {"block_m": c["block_m"]}):
+        out = matmul(xdev, v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter), precision_config=pc,
+                     betas=dev(betas), gammas=dev(gammas), fused_activation=fa, c=out_init)
+    ref = ref.to(out_dtype)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    assert_close(ref, out.cpu(), maxtol=3e-2, verbose=False)

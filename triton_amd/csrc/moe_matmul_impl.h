@@ -502,8 +502,20 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
                                                                         0x00020000);
       const int n_dw = (BLOCK_N * G + 3) / 4;
-      for (int i = tid; i < n_dw; i += 256)
-        ((uint32_t *)lds_sc)[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);
+      const int avail = tile_cols * G;
+      for (int i = tid; i < n_dw; i += 256) {
+        uint32_t v;
+        if (i * 4 + 4 <= avail || i * 4 >= avail) {
+          v = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);  // whole, or wholly outside (zeros)
+        } else {
+          // the dword that straddles the end of the scales: a dword load that is partly out of range returns
+          // zeros for all four bytes, so the bytes inside are fetched one by one
+          v = 0;
+          for (int b = 0; i * 4 + b < avail; ++b)
+            v |= (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(rs, i * 4 + b, 0, 0) << (8 * b);
+        }
+        ((uint32_t *)lds_sc)[i] = v;
+      }
     }
   }
   // offset of a column's scales inside the tile's image (LDS) or, without staging, from the expert's first scale
