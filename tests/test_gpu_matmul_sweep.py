@@ -2,6 +2,7 @@
 activation type x row-block size x weight-scale layout x gather / scatter / betas / gammas / bias type x output type x
 SwiGLU, on ragged problems with random (often empty or tiny) slices and odd sizes.  Every case goes through the C
 ABI and is compared with the CPU oracle (rtol = atol = 1e-2 on the scale of the outputs, see `check`)."""
+import os
 import random
 
 import pytest
@@ -42,7 +43,8 @@ def make_case(seed):
     return c
 
 
-@pytest.mark.parametrize("seed", range(60))
+# TAMD_SWEEP_CASES widens the sweep for exploration; the default keeps the suite short
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TAMD_SWEEP_CASES", "60"))))
 def test_sweep(seed, device):
     c = make_case(seed)
     print("case", c, flush=True)
@@ -104,6 +106,87 @@ def test_sweep(seed, device):
     with scoped_opt_flags_constraints({} if c["block_m"] is None else {"block_m": c["block_m"]}):
         out = matmul(xdev, v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter), precision_config=pc,
                      betas=dev(betas), gammas=dev(gammas), fused_activation=fa, c=out_init)
+    ref = ref.to(out_dtype)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    assert_close(ref, out.cpu(), maxtol=3e-2, verbose=False)
+
+
+def make_dense_case(seed):
+    rng = random.Random(1000 + seed)
+    c = dict(seed=seed)
+    c["weights"] = rng.choice(["mxfp4", "mxfp4", "w16_k", "w16_n"])
+    c["kind"] = rng.choice(["bf16", "f16"]) if c["weights"] != "mxfp4" else KINDS[seed % len(KINDS)]
+    c["batch"] = rng.choice([0, 0, 2, 3])  # 0: plain [M, K] x [K, N]
+    c["M"] = rng.choice([1, 7, 16, 17, 40, 64, 100, 130, 257, 300])
+    c["K"] = 32 * rng.choice([1, 2, 3, 5, 8, 13, 16, 32, 45, 64])
+    c["N"] = 2 * rng.choice([4, 8, 16, 33, 100, 128, 131, 264, 300, 520])
+    c["split_k"] = rng.choice([1, 1, 1, 2, 3])
+    c["cdna4"] = c["weights"] == "mxfp4" and c["split_k"] == 1 and rng.random() < 0.4
+    c["bias"] = rng.choice([None, torch.float32, torch.bfloat16])
+    c["act"] = rng.random() < 0.4
+    c["alpha"] = rng.choice([None, 0.5])
+    c["out"] = rng.choice([None, torch.float32]) if c["kind"] in ("bf16", "f16") else rng.choice([torch.bfloat16, torch.float32])
+    if c["weights"] != "mxfp4" and c["split_k"] > 1 and c["K"] % 64:
+        c["split_k"] = 1
+    return c
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TAMD_SWEEP_CASES", "60"))))
+def test_sweep_dense_and_batched(seed, device):
+    """Plain and batched problems: MXFP4 and unquantised 16-bit weights (either axis contiguous), split-K, out_alpha."""
+    c = make_dense_case(seed)
+    print("case", c, flush=True)
+    torch.manual_seed(seed)
+    B, M, K, N = c["batch"], c["M"], c["K"], c["N"]
+    lead = (B, ) if B else ()
+    x0 = torch.randn(*lead, M, K)
+    w = torch.randn(*lead, K, N) * 0.05
+    bias = None if c["bias"] is None else torch.randn(*lead, N).to(c["bias"])
+    kw = dict(out_alpha=c["alpha"], fused_swiglu=(1.702, 7.0) if c["act"] else None)
+    kind = c["kind"]
+    flex = FlexCtx()
+    a_mx = None
+    if c["weights"] == "mxfp4":
+        v, s = downcast_to_mxfp(w.to(device), torch.uint8, axis=-2)
+        rv, rs = downcast_to_mxfp_ref(w, torch.uint8, axis=-2)
+        assert torch.equal(v.cpu(), rv) and torch.equal(s.cpu(), rs)
+        wdev, kw["b_mx_scale"] = v, rs
+        sc = convert_layout(wrap_torch_tensor(s), CDNA4MXScaleLayout()) if c["cdna4"] else s
+        wref = rv
+    else:
+        dt = torch.bfloat16 if kind == "bf16" else torch.float16
+        wref = w.to(dt)
+        wdev = wref.to(device)
+        if c["weights"] == "w16_k":
+            wdev = wdev.transpose(-1, -2).contiguous().transpose(-1, -2)  # unit stride along K
+        sc = None
+    if kind in ("bf16", "f16"):
+        dt = torch.bfloat16 if kind == "bf16" else torch.float16
+        xq = x0.to(dt)
+        xdev = xq.to(device)
+        ref = MR.matmul_ref(xq, wref, bias, **kw)
+        out_dtype = c["out"] or dt
+    elif kind in ("e4m3", "e5m2"):
+        fp8 = torch.float8_e4m3fn if kind == "e4m3" else torch.float8_e5m2
+        x_scale = (x0.abs().max() / 448.0).reshape(1).float()
+        xq = (x0 / x_scale).to(fp8)
+        xdev = xq.to(device)
+        flex = FlexCtx(lhs_data=InFlexData(dtype=fp8, scale=x_scale.to(device)))
+        ref = MR.matmul_ref(xq, wref, bias, a_flex_scale=x_scale, **kw)
+        out_dtype = c["out"]
+    else:
+        xdev, a_mx = downcast_to_mxfp(x0.to(device), torch.float8_e4m3fn, axis=-1)
+        rq, rxs = downcast_to_mxfp_ref(x0, torch.float8_e4m3fn, axis=-1)
+        assert torch.equal(xdev.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(a_mx.cpu(), rxs)
+        ref = MR.matmul_ref(rq, wref, bias, a_mx_scale=rxs, **kw)
+        out_dtype = c["out"]
+    pc = PrecisionConfig(a_mx_scale=a_mx, a_microblock_size=32 if a_mx is not None else None, b_mx_scale=sc,
+                         b_microblock_size=32 if sc is not None else None, out_dtype=c["out"], flex_ctx=flex)
+    fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if c["act"] else None
+    with scoped_opt_flags_constraints({} if c["split_k"] == 1 else {"split_k": c["split_k"]}):
+        out = matmul(xdev, wdev, None if bias is None else bias.to(device), precision_config=pc, out_alpha=c["alpha"],
+                     fused_activation=fa)
+    assert out.dtype == out_dtype and tuple(out.shape) == (*lead, M, N // 2 if c["act"] else N)
     ref = ref.to(out_dtype)
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
     assert_close(ref, out.cpu(), maxtol=3e-2, verbose=False)

@@ -164,6 +164,11 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         b_scale = None
     a = flex.lhs_data.reinterpret(a)
     w = flex.rhs_data.reinterpret(b.storage.data)
+    if b.dtype != FP4 and w.stride(-1) == 1 and (w.shape[-1] * w.element_size()) % 16 != 0 \
+            and (w.shape[-2] * w.element_size()) % 16 == 0:
+        # unquantised weights with unit stride along N whose rows do not start on 16-byte boundaries: the kernel copies
+        # 16 bytes at a time, so they are laid out with unit stride along K instead (same values)
+        w = w.transpose(-1, -2).contiguous().transpose(-1, -2)
     _lib.require_gpu(a, "a")
     _lib.require_gpu(w, "b")
     assert a.stride(-1) == 1 or a.shape[-1] == 1, "a must be contiguous along K"
