@@ -128,9 +128,9 @@ def upcast_from_mxfp(tensor: torch.Tensor, scale: torch.Tensor, target_dtype: to
     out = torch.empty(out_shape, dtype=target_dtype, device=tensor.device)
     if out.numel() > 0:
         if tensor.stride(axis) != 1 or _as_3d(tensor, axis) is None:
-            tensor = tensor.transpose(axis, -1).contiguous().transpose(axis, -1)
+            tensor = tensor.movedim(axis, -1).contiguous().movedim(-1, axis)  # unit stride along axis, the rest in order
         if scale.stride(axis) != 1 or _as_3d(scale, axis) is None:
-            scale = scale.transpose(axis, -1).contiguous().transpose(axis, -1)
+            scale = scale.movedim(axis, -1).contiguous().movedim(-1, axis)
         vv, sv, ov = _as_3d(tensor, axis), _as_3d(scale, axis), _as_3d(out, axis)
         nb, _, nr = ov[0], ov[1], ov[2]
         dsl, dsr = ov[4], ov[5]
