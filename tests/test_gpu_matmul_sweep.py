@@ -1,7 +1,8 @@
 """GPU parity: a seeded sweep over combinations the hand-written cases of test_gpu_matmul.py do not enumerate --
 activation type x row-block size x weight-scale layout x gather / scatter / betas / gammas / bias type x output type x
 SwiGLU, on ragged problems with random (often empty or tiny) slices and odd sizes.  Every case goes through the C
-ABI and is compared with the CPU oracle (rtol = atol = 1e-2 on the scale of the outputs, see `check`)."""
+ABI and is compared with the CPU oracle (rtol = atol = 1e-2, plus the reference's own error measure).  For exploration,
+TAMD_SWEEP_CASES=<n> widens every sweep and TAMD_SWEEP_LONG_K=1 adds K up to 8192 to the ragged one."""
 import os
 import random
 
@@ -28,7 +29,7 @@ def make_case(seed):
     c = dict(seed=seed)
     c["kind"] = KINDS[seed % len(KINDS)]
     c["E"] = rng.choice([1, 2, 5, 9])
-    c["K"] = 32 * rng.choice([1, 2, 3, 5, 10, 13, 32, 45])
+    c["K"] = 32 * rng.choice([1, 2, 3, 5, 10, 13, 32, 45] + ([90, 128, 129, 160, 256] if os.environ.get("TAMD_SWEEP_LONG_K") else []))
     c["N"] = 2 * rng.choice([8, 16, 33, 100, 128, 131, 264, 300])
     c["sizes"] = [rng.choice([0, 1, 2, 15, 16, 17, 31, 33, 64, 100, 129, 161, 260]) for _ in range(c["E"])]
     if sum(c["sizes"]) == 0:
