@@ -183,7 +183,7 @@ typedef struct tamd_matmul_args {
   float out_alpha; /* 1.0 when unused */
   /* output [rows_out, N_out], unit stride along N */
   void *y;
-  int y_dtype; /* TAMD_BF16 / TAMD_F16 / TAMD_F32 / TAMD_FP8_E4M3 */
+  int y_dtype; /* TAMD_BF16 / TAMD_F16 / TAMD_F32 / TAMD_FP8_E4M3 / TAMD_FP8_E5M2 */
   int64_t y_stride_m;
   /* problem */
   int M; /* rows to compute (len(gather_indx) or rows of x); per expert if not ragged */
@@ -211,7 +211,7 @@ typedef struct tamd_matmul_args {
   /* flexpoint output (numerics_details/flexpoint.py:137-188, float_to_flex / update_scale): the result is
    * multiplied by 1 / *y_expected_scale before the cast (and clamped to the finite range of y_dtype when
    * y_saturate_inf); max|result| / max_finite(y_dtype) + 1e-30 is folded into *y_actual_scale by atomic max
-   * (NaN counts as +inf).  Either pointer may be NULL.  y_dtype may then also be TAMD_FP8_E4M3. */
+   * (NaN counts as +inf).  Either pointer may be NULL.  y_dtype may then also be TAMD_FP8_E4M3 / TAMD_FP8_E5M2. */
   const float *y_expected_scale;
   float *y_actual_scale;
   int y_saturate_inf;

@@ -322,10 +322,11 @@ def test_decode_shape_of_the_baseline(device):
 # ---------------------------------------------------------------------------- flexpoint (fp8) output
 
 
-def test_fp8_output_conversion_is_exact(device):
+@pytest.mark.parametrize("fp8,top", [(torch.float8_e4m3fn, 6.0), (torch.float8_e5m2, 11.0)])
+def test_fp8_output_conversion_is_exact(fp8, top, device):
     """One-hot activations times a per-row gate weight give single float32 products deq(W)[k, n] * gamma[r]: the
-    fp8 output must equal torch's own float32 -> float8_e4m3fn cast of them bit for bit (round to nearest even,
-    subnormals, NaN beyond the range without saturation, the largest finite value with it)."""
+    fp8 output must equal torch's own float32 -> fp8 cast of them bit for bit (round to nearest even, subnormals,
+    beyond the range NaN for e4m3fn and infinity for e5m2 without saturation, the largest finite value with it)."""
     from triton_amd.matmul import OutFlexData
     torch.manual_seed(0)
     K, N, M = 64, 256, 64
@@ -334,20 +335,22 @@ def test_fp8_output_conversion_is_exact(device):
     from oracle.mxfp_ref import upcast_from_mxfp_ref
     deq = upcast_from_mxfp_ref(rv, rs, torch.float32, axis=0)
     x = torch.eye(K, dtype=torch.bfloat16)[:M]
-    gammas = torch.exp(torch.linspace(-12, 6, M)).float()
+    gammas = torch.exp(torch.linspace(-12 - top / 2, top, M)).float()
+    max_q = torch.finfo(fp8).max
     for saturate in (False, True):
         actual = torch.zeros(1, device=device)
-        flex = FlexCtx(out_data=OutFlexData(torch.float8_e4m3fn, torch.ones(1, device=device), actual, None))
-        pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, flex_ctx=flex,
+        flex = FlexCtx(out_data=OutFlexData(fp8, torch.ones(1, device=device), actual, None))
+        pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=fp8, flex_ctx=flex,
                              flexpoint_saturate_inf=saturate)
         out = matmul(x.to(device), v, None, precision_config=pc, gammas=gammas.to(device))
-        assert out.dtype == torch.float8_e4m3fn
+        assert out.dtype == fp8
         prod = deq[:M] * gammas[:, None]
-        want = (prod.clamp(-448, 448) if saturate else prod).to(torch.float8_e4m3fn)
+        assert prod.abs().max() > 1.2 * max_q  # the range is exceeded somewhere
+        want = (prod.clamp(-max_q, max_q) if saturate else prod).to(fp8)
         # a -0.0 weight summed with the +0.0 products of the other K positions is +0.0: ignore the sign of zero
         pos_zero = lambda t: torch.where(t == 0x80, torch.zeros_like(t), t)
         assert torch.equal(pos_zero(out.cpu().view(torch.uint8)), pos_zero(want.view(torch.uint8)))
-        assert actual.item() == pytest.approx(float(prod.abs().max()) / 448.0, rel=1e-6)
+        assert actual.item() == pytest.approx(float(prod.abs().max()) / max_q, rel=1e-6)
 
 
 @pytest.mark.parametrize("block_m", [16, 128])

@@ -247,15 +247,17 @@ def test_sweep_quantised_outputs(seed, device):
     if mode == "flex":
         expected = torch.tensor([2.0**rng.choice([-6, -4, 0])], device=device)
         actual = torch.zeros(1, device=device)
-        flex = FlexCtx(lhs_data=lhs, out_data=OutFlexData(torch.float8_e4m3fn, expected, actual, None))
-        y8 = run(PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, flex_ctx=flex,
+        fp8 = torch.float8_e4m3fn if seed % 3 else torch.float8_e5m2
+        max_q = torch.finfo(fp8).max
+        flex = FlexCtx(lhs_data=lhs, out_data=OutFlexData(fp8, expected, actual, None))
+        y8 = run(PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=fp8, flex_ctx=flex,
                                  flexpoint_saturate_inf=True)).cpu()
-        want = (y32 / expected.item()).clamp(-448, 448).to(torch.float8_e4m3fn)
+        want = (y32 / expected.item()).clamp(-max_q, max_q).to(fp8)
         assert torch.equal(y8.view(torch.uint8), want.view(torch.uint8))
         # rows dropped by the scatter are computed all the same and count for the maximum
-        assert actual.item() >= MR.actual_scale_ref(y32, torch.float8_e4m3fn).item() * (1 - 1e-6)
+        assert actual.item() >= MR.actual_scale_ref(y32, fp8).item() * (1 - 1e-6)
         if not do_scatter:
-            assert actual.item() == pytest.approx(MR.actual_scale_ref(y32, torch.float8_e4m3fn).item(), rel=1e-6)
+            assert actual.item() == pytest.approx(MR.actual_scale_ref(y32, fp8).item(), rel=1e-6)
     else:
         c_scale = torch.zeros((M, -(-n_out // 32)), dtype=torch.uint8, device=device)
         pc = PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=torch.float8_e4m3fn, c_mx_scale=c_scale,

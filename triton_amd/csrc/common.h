@@ -37,10 +37,22 @@ TAMD_DEVICE uint32_t f32_to_e4m3_bits(float f, bool saturate) {
   return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false) & 0xFFu;
 }
 
+// float32 -> OCP e5m2 byte, round to nearest even.  Magnitudes that round beyond 57344 (>= 61440) give infinity
+// (or the largest finite code when saturating); NaN stays NaN.
+TAMD_DEVICE uint32_t f32_to_e5m2_bits(float f, bool saturate) {
+  const uint32_t u = f32_to_bits(f), sign = (u >> 24) & 0x80u, mag = u & 0x7FFFFFFFu;
+  if (mag > 0x7F800000u) return sign | 0x7Fu;
+  if (mag >= 0x47700000u) return sign | (saturate ? 0x7Bu : 0x7Cu);  // 61440.0f
+  return (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(f, f, 0, false) & 0xFFu;
+}
+TAMD_DEVICE uint32_t f32_to_fp8_bits(float f, int dt) {
+  return dt == TAMD_FP8_E5M2 ? f32_to_e5m2_bits(f, false) : f32_to_e4m3_bits(f, false);
+}
+
 // Largest finite value of an output type, and the running |x| maximum kept as float bits so that NaN
 // (above +inf as an integer) survives the maximum (flexpoint.py:119-146 of the reference).
 TAMD_DEVICE float max_finite_of(int dt) {
-  return dt == TAMD_FP8_E4M3 ? 448.0f : (dt == TAMD_F16 ? 65504.0f : (dt == TAMD_BF16 ? 3.3895313892515355e38f : 3.4028234663852886e38f));
+  return dt == TAMD_FP8_E4M3 ? 448.0f : dt == TAMD_FP8_E5M2 ? 57344.0f : (dt == TAMD_F16 ? 65504.0f : (dt == TAMD_BF16 ? 3.3895313892515355e38f : 3.4028234663852886e38f));
 }
 TAMD_DEVICE uint32_t absmax_bits(uint32_t run, float v) {
   const uint32_t b = f32_to_bits(v) & 0x7FFFFFFFu;

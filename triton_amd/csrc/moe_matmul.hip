@@ -23,9 +23,9 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
   if (!a.x || !a.w || !a.y) return TAMD_E_INVALID;
   if (a.activation != TAMD_ACT_NONE && a.activation != TAMD_ACT_SWIGLU) return TAMD_E_INVALID;
   if (a.activation == TAMD_ACT_SWIGLU && (a.N % 2) != 0) return TAMD_E_INVALID;
-  if (a.y_dtype == TAMD_FP8_E5M2) return TAMD_E_UNSUPPORTED;
   if (a.y_mx_scale && (a.y_dtype != TAMD_FP8_E4M3 || a.y_expected_scale || a.y_actual_scale)) return TAMD_E_UNSUPPORTED;
-  if (a.y_dtype != TAMD_BF16 && a.y_dtype != TAMD_F16 && a.y_dtype != TAMD_F32 && a.y_dtype != TAMD_FP8_E4M3)
+  if (a.y_dtype != TAMD_BF16 && a.y_dtype != TAMD_F16 && a.y_dtype != TAMD_F32 && a.y_dtype != TAMD_FP8_E4M3 &&
+      a.y_dtype != TAMD_FP8_E5M2)
     return TAMD_E_INVALID;
   if (a.bias && a.bias_dtype != TAMD_F32 && a.bias_dtype != TAMD_BF16 && a.bias_dtype != TAMD_F16)
     return TAMD_E_INVALID;

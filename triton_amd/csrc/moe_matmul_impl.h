@@ -253,7 +253,7 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
   const int out_col0 = ACT == TAMD_ACT_SWIGLU ? col0 / 2 : col0;
   const int tile_out0 = ACT == TAMD_ACT_SWIGLU ? t.n0 / 2 : t.n0;
   const bool has_limit = a.act_has_limit != 0;
-  const int osz = ydt == TAMD_F32 ? 4 : (ydt == TAMD_FP8_E4M3 ? 1 : 2);  // bytes per output
+  const int osz = ydt == TAMD_F32 ? 4 : (is_fp8(ydt) ? 1 : 2);  // bytes per output
   const bool staged = osz < 4;
   // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
   const float inv_expected = (FLEX && a.y_expected_scale) ? 1.0f / *a.y_expected_scale : 1.0f;
@@ -262,7 +262,7 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
   const bool track_max = FLEX && a.y_actual_scale != nullptr;
   uint32_t amax = 0;
   auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
-    return ydt == TAMD_BF16 ? f32_to_bf16_bits(v) : (ydt == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_e4m3_bits(v, false));
+    return ydt == TAMD_BF16 ? f32_to_bf16_bits(v) : (ydt == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_fp8_bits(v, ydt));
   };
   // without per-row factors bias * beta * out_alpha is one value per column
   float bias_a[NF];

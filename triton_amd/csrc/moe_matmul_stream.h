@@ -177,10 +177,10 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
                                                            : (a.bias_dtype == TAMD_BF16 ? bits_to_f32(raw << 16)
                                                                                         : f16_bits_to_f32((uint16_t)raw)));
     };
-    const int osz = a.y_dtype == TAMD_F32 ? 4 : (a.y_dtype == TAMD_FP8_E4M3 ? 1 : 2);
+    const int osz = a.y_dtype == TAMD_F32 ? 4 : (is_fp8(a.y_dtype) ? 1 : 2);
     auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
       return a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(v) & 0xFFFFu
-                                    : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) & 0xFFFFu : f32_to_e4m3_bits(v, false));
+                                    : (a.y_dtype == TAMD_F16 ? f32_to_f16_bits(v) & 0xFFFFu : f32_to_fp8_bits(v, a.y_dtype));
     };
     // flexpoint output: scale by 1 / expected, optionally clamp, and track max|result| for the actual scale
     const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;

@@ -193,8 +193,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
             raise NotImplementedError("MXFP8 output needs float8_e4m3fn values")
         if flex.out_data.expected_scale is not None or flex.out_data.actual_scale is not None:
             raise NotImplementedError("flexpoint output scales together with MX output scales are not built")
-    if out_dtype.itemsize == 1 and out_dtype != torch.float8_e4m3fn:
-        raise NotImplementedError(f"{out_dtype} outputs are not built (float8_e4m3fn is)")
+    if out_dtype.itemsize == 1 and out_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
+        raise NotImplementedError(f"{out_dtype} outputs are not built (float8_e4m3fn and float8_e5m2 are)")
     rows_out = M
     if gather_indx is not None:
         rows_out = gather_indx.shape[0]
