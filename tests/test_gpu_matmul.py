@@ -844,3 +844,37 @@ def test_mxfp8_weights(fp8, ragged, device):
         out = matmul(x.to(device), v[0], bias[0].to(device), precision_config=pc)
         ref = MR.matmul_ref(x, rv[0], bias[0], b_mx_scale=rs[0])
     check(out, ref)
+
+
+@pytest.mark.parametrize("fp8", [torch.float8_e5m2, torch.float8_e4m3fn])
+@pytest.mark.parametrize("mode", ["plain", "ragged", "batched"])
+def test_fp8_activations_times_fp8_weights(fp8, mode, device):
+    """float8 x float8 with per-tensor flex scales on both operands (tests/test_matmul.py:150-154 of the reference),
+    float32 output against the oracle, and the same problem with an fp8 flexpoint output against the cast of that."""
+    from triton_amd.matmul import OutFlexData
+    torch.manual_seed(4)
+    E, K, N = (3, 320, 264)
+    sizes = torch.tensor([40, 0, 130], dtype=torch.int32)
+    M = int(sizes.sum()) if mode == "ragged" else 70
+    lead = {"plain": (), "ragged": (), "batched": (E, )}[mode]
+    x0 = torch.randn(*lead, M, K)
+    w0 = torch.randn(*(lead if mode != "ragged" else (E, )), K, N) * 0.05
+    bias = torch.randn(*(lead if mode != "ragged" else (E, )), N)
+    x_scale, w_scale = (x0.abs().max() / 400).reshape(1), (w0.abs().max() / 400).reshape(1)
+    x8, w8 = (x0 / x_scale).to(fp8), (w0 / w_scale).to(fp8)
+    flex = FlexCtx(lhs_data=InFlexData(dtype=fp8, scale=x_scale.to(device)), rhs_data=InFlexData(dtype=fp8, scale=w_scale.to(device)))
+    md = make_ragged_tensor_metadata(sizes.to(device), M) if mode == "ragged" else None
+    out = matmul(x8.to(device), w8.to(device), bias.to(device), md,
+                 precision_config=PrecisionConfig(flex_ctx=flex, out_dtype=torch.float32))
+    ref = MR.matmul_ref(x8, w8, bias, slice_sizes=sizes if mode == "ragged" else None, a_flex_scale=x_scale,
+                        b_flex_scale=w_scale)
+    check(out, ref)
+    expected = torch.tensor([0.25], device=device)
+    actual = torch.zeros(1, device=device)
+    flex8 = FlexCtx(lhs_data=flex.lhs_data, rhs_data=flex.rhs_data, out_data=OutFlexData(fp8, expected, actual, None))
+    out8 = matmul(x8.to(device), w8.to(device), bias.to(device), md,
+                  precision_config=PrecisionConfig(flex_ctx=flex8, flexpoint_saturate_inf=True))
+    assert out8.dtype == fp8  # the output type defaults to the activations' type
+    max_q = torch.finfo(fp8).max
+    assert torch.equal(out8.cpu().view(torch.uint8), (out.cpu() / 0.25).clamp(-max_q, max_q).to(fp8).view(torch.uint8))
+    assert actual.item() == pytest.approx(float(out.abs().max()) / max_q, rel=1e-6)

@@ -164,6 +164,13 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         b_scale = None
     a = flex.lhs_data.reinterpret(a)
     w = flex.rhs_data.reinterpret(b.storage.data)
+    a_dtype = a.dtype  # the type the output defaults to
+    fp8_types = (torch.float8_e4m3fn, torch.float8_e5m2)
+    if b.dtype != FP4 and w.dtype in fp8_types and a.dtype in fp8_types and a_mx_scale is None:
+        # fp8 x fp8 with per-tensor scales (tests/test_matmul.py:150-154 of the reference): every fp8 number is a
+        # bfloat16 number, so both operands are widened (exactly) and multiplied by the kernel for 16-bit weights; the
+        # flex scales enter in its epilogue as they do for any other pair of types
+        a, w = a.to(torch.bfloat16), w.to(torch.bfloat16)
     if b.dtype != FP4 and w.stride(-1) == 1 and (w.shape[-1] * w.element_size()) % 16 != 0 \
             and (w.shape[-2] * w.element_size()) % 16 == 0:
         # unquantised weights with unit stride along N whose rows do not start on 16-byte boundaries: the kernel copies
@@ -186,7 +193,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
     # microscaled activations stand for bf16 numbers (the reference dequantises them to bf16, matmul.py:772-778)
-    out_dtype = precision_config.out_dtype or (torch.bfloat16 if a_mx_scale is not None else a.dtype)
+    out_dtype = precision_config.out_dtype or (torch.bfloat16 if a_mx_scale is not None else a_dtype)
     if mx_out:
         out_dtype = precision_config.out_dtype or (c.dtype if c is not None else torch.float8_e4m3fn)
         if out_dtype != torch.float8_e4m3fn:
