@@ -28,6 +28,45 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const void *__restrict__ a,
   }
 }
 
+// Four outputs (eight interleaved inputs) per thread: rows and pitches aligned so that a thread's inputs are one or
+// two 16-byte loads and its outputs one 8- or 16-byte store.
+template <int DT>
+__global__ __launch_bounds__(256) void swiglu_vec4_kernel(const void *__restrict__ a, int64_t M, int64_t N,
+                                                          int64_t a_stride, void *__restrict__ out, int64_t o_stride,
+                                                          float alpha, float limit, int has_limit) {
+  const int64_t nq = N / 4, total = M * nq;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / nq, n = (i - m * nq) * 4;
+    float v[8];
+    if constexpr (DT == TAMD_F32) {
+      const float4 lo = *(const float4 *)((const float *)a + m * a_stride + 2 * n);
+      const float4 hi = *(const float4 *)((const float *)a + m * a_stride + 2 * n + 4);
+      v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    } else {
+      const uint4 q = *(const uint4 *)((const uint16_t *)a + m * a_stride + 2 * n);
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = DT == TAMD_BF16 ? bf16_bits_to_f32(w[j] & 0xFFFFu) : f16_bits_to_f32(w[j] & 0xFFFFu);
+        v[2 * j + 1] = DT == TAMD_BF16 ? bf16_bits_to_f32(w[j] >> 16) : f16_bits_to_f32(w[j] >> 16);
+      }
+    }
+    float o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = swiglu_f32(v[2 * j], v[2 * j + 1], alpha, limit, has_limit != 0);
+    if constexpr (DT == TAMD_F32) {
+      *(float4 *)((float *)out + m * o_stride + n) = make_float4(o[0], o[1], o[2], o[3]);
+    } else {
+      uint32_t w[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        w[j] = DT == TAMD_BF16 ? ((f32_to_bf16_bits(o[2 * j]) & 0xFFFFu) | (f32_to_bf16_bits(o[2 * j + 1]) << 16))
+                               : ((f32_to_f16_bits(o[2 * j]) & 0xFFFFu) | (f32_to_f16_bits(o[2 * j + 1]) << 16));
+      *(uint2 *)((uint16_t *)out + m * o_stride + n) = make_uint2(w[0], w[1]);
+    }
+  }
+}
+
 // x [S0, R, S1] -> y [S0, S1].  VEC elements of the inner axis per thread when
 // the inner stride is 1 and everything is 16-byte aligned.
 template <int XDT, int YDT, int VEC>
@@ -100,6 +139,29 @@ __global__ __launch_bounds__(256) void reduce_kernel(const void *__restrict__ x,
         acc[j] += t;
       }
     }
+    if constexpr (VEC > 1) {
+      // the vector form has S1 % VEC == 0: with a dense, aligned output row the VEC results leave as 16-byte stores
+      // (element-wise 2-byte stores at a 16-byte lane pitch use an eighth of every write they cause)
+      constexpr int YS = YDT == TAMD_F32 ? 4 : 2;
+      uint8_t *yp = (uint8_t *)y + (s0 * ys0 + c0) * YS;
+      constexpr int ALIGN = VEC * YS < 16 ? VEC * YS : 16;
+      if (ys1 == 1 && (((uintptr_t)yp) & (ALIGN - 1)) == 0) {
+        if constexpr (YDT == TAMD_F32) {
+#pragma unroll
+          for (int j = 0; j < VEC; j += 4) *(float4 *)(yp + j * 4) = make_float4(acc[j], acc[j + 1], acc[j + 2], acc[j + 3]);
+        } else {
+          uint32_t w[VEC / 2];
+#pragma unroll
+          for (int j = 0; j < VEC / 2; ++j) {
+            if constexpr (YDT == TAMD_BF16) w[j] = (f32_to_bf16_bits(acc[2 * j]) & 0xFFFFu) | (f32_to_bf16_bits(acc[2 * j + 1]) << 16);
+            else w[j] = (f32_to_f16_bits(acc[2 * j]) & 0xFFFFu) | (f32_to_f16_bits(acc[2 * j + 1]) << 16);
+          }
+          if constexpr (VEC == 8) *(uint4 *)yp = make_uint4(w[0], w[1], w[2], w[3]);
+          else *(uint2 *)yp = make_uint2(w[0], w[1]);
+        }
+        continue;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
       if (c0 + j < S1) store_from_f32<YDT>(y, s0 * ys0 + (c0 + j) * ys1, acc[j]);
@@ -158,6 +220,19 @@ extern "C" int tamd_swiglu(const void *a, int dtype, int64_t M, int64_t N_out, i
   if (M == 0 || N_out == 0) return 0;
   if (!a || !out) return TAMD_E_INVALID;
   hipStream_t st = (hipStream_t)stream;
+  const int esz = dtype == TAMD_F32 ? 4 : 2;
+  if (N_out % 4 == 0 && aligned(a, 16) && aligned(out, 16) && (a_stride_m * esz) % 16 == 0 && (out_stride_m * esz) % 16 == 0 &&
+      (dtype == TAMD_F32 || dtype == TAMD_BF16 || dtype == TAMD_F16)) {
+    int64_t vblocks = (M * (N_out / 4) + 255) / 256;
+    if (vblocks > 256 * 64) vblocks = 256 * 64;
+    if (dtype == TAMD_F32)
+      swiglu_vec4_kernel<TAMD_F32><<<dim3((unsigned)vblocks), 256, 0, st>>>(a, M, N_out, a_stride_m, out, out_stride_m, alpha, limit, has_limit);
+    else if (dtype == TAMD_BF16)
+      swiglu_vec4_kernel<TAMD_BF16><<<dim3((unsigned)vblocks), 256, 0, st>>>(a, M, N_out, a_stride_m, out, out_stride_m, alpha, limit, has_limit);
+    else
+      swiglu_vec4_kernel<TAMD_F16><<<dim3((unsigned)vblocks), 256, 0, st>>>(a, M, N_out, a_stride_m, out, out_stride_m, alpha, limit, has_limit);
+    return launch_status();
+  }
   int64_t blocks = (M * N_out + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
   switch (dtype) {
