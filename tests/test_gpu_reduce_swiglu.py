@@ -75,3 +75,17 @@ def test_reduce_mxfp8_in_and_out(shape, dim, mask_mode, use_scale, use_flex, dev
                               x_flex_scale=None)
     assert yv.dtype == torch.float8_e4m3fn and torch.equal(ys.cpu(), rs)
     assert torch.equal(yv.cpu().view(torch.uint8), rv.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("shape,dim", [((8, 4096, 256), 1), ((2048, 40), 0), ((3, 1000, 7), 1)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_reduce_long_axis(shape, dim, dtype, device):
+    """A long reduced axis over few outputs is summed in chunks (float32 partial sums): same sum up to the order of
+    the additions."""
+    torch.manual_seed(0)
+    x = torch.randn(shape).to(dtype)
+    y, _ = reduce(x.to(device), dim)
+    ref = MR.reduce_ref(x, dim)
+    assert y.dtype == dtype and tuple(y.shape) == tuple(ref.shape)
+    tol = dict(rtol=1e-2, atol=5e-1) if dtype != torch.float32 else dict(rtol=1e-4, atol=1e-3)
+    torch.testing.assert_close(y.cpu().float(), ref.float(), **tol)

@@ -60,6 +60,14 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
     R = x.shape[dim]
     if not x.is_contiguous():
         x = x.contiguous()
+    if mask is None and scale is None and y is None and R >= 512 and lead * tail <= (1 << 18):
+        # a long axis over few outputs: a thread of the kernel walks the whole axis, so it is cut into chunks that
+        # are summed side by side (float32 partial sums), then the chunks are summed
+        chunks = next((c for c in (64, 32, 16, 8) if R % c == 0), 0)
+        if chunks:
+            part, _ = reduce(x.view(lead, chunks, R // chunks, tail), 2, y_dtype=torch.float32)
+            out, _ = reduce(part, 1, y_dtype=y_dtype or x.dtype)
+            return out.view([*x.shape[:dim], *x.shape[dim + 1:]]), None
     x3 = x.view(lead, R, tail)
 
     def to3(t):
