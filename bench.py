@@ -25,7 +25,7 @@ PEAK_MXFP4_TFLOPS = 10100.0
 
 # HBM bytes per launch of the dominant kernel (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00 KiB from rocprofv3 --pmc,
 # factors from the hbm_copy workload).  Counters cannot be read from inside this process; re-measure after kernel changes.
-MEASURED_TRAFFIC = {"fc1_prefill": 1617191639, "fc1_decode": 976166507, "fc2_combine": 1496500221}
+MEASURED_TRAFFIC = {"fc1_prefill": 1611457371, "fc1_decode": 976176743, "fc2_combine": 1497319402}
 
 WORKLOADS = {
     # name: (T, E, k, K, N, swiglu)
