@@ -265,15 +265,19 @@ __global__ __launch_bounds__(256) void upcast_cols_kernel(
     const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
     int64_t csb, int64_t csr, void *__restrict__ dst, int64_t nb, int64_t G, int64_t nr, int64_t dsb,
     int64_t dsl) {
+  // a workgroup covers 8 consecutive groups of 32 column sets: the 8 lanes that share a column set read 8 x 16
+  // consecutive bytes of each of its columns (one 128-byte line) and 8 consecutive scale bytes.  The grid is
+  // ceil(n_rv / 32) * ceil(G / 8) * nb workgroups (launch_upcast).
   int64_t n_rv = (nr + NV - 1) / NV;
-  int64_t blocks_r = (n_rv + 255) / 256;
+  int64_t blocks_r = (n_rv + 31) / 32;
+  int64_t g_chunks = (G + 7) / 8;
   int64_t bid = blockIdx.x;
   int64_t br = bid % blocks_r;
   int64_t t = bid / blocks_r;
-  int64_t g = t % G;
-  int64_t b = t / G;
-  int64_t rv = br * 256 + threadIdx.x;
-  if (rv >= n_rv) return;
+  int64_t g = (t % g_chunks) * 8 + threadIdx.x % 8;
+  int64_t b = t / g_chunks;
+  int64_t rv = br * 32 + threadIdx.x / 8;
+  if (rv >= n_rv || g >= G || b >= nb) return;
   int64_t r0 = rv * NV;
   uint4 code[NV];
   float mult[NV];
@@ -364,12 +368,12 @@ int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsl * ES) % 16 == 0;
   if (vec) {
-    int64_t blocks = ((nr / NV + 255) / 256) * G * nb;
+    int64_t blocks = ((nr / NV + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
     upcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
                                                                       nr, dsb, dsl);
   } else {
-    int64_t blocks = ((nr + 255) / 256) * G * nb;
+    int64_t blocks = ((nr + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
     upcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
                                                                      nr, dsb, dsl);
