@@ -154,15 +154,19 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
     const void *__restrict__ src, int64_t nb, int64_t G, int64_t nr, int64_t ssb, int64_t ssl,
     uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
     int64_t csr, int mode) {
+  // a workgroup covers 8 consecutive groups of 32 column sets: the 8 lanes that share a column set write 8 x 16
+  // consecutive bytes of codes of each of its columns (one 128-byte line) and 8 consecutive scale bytes.  The
+  // grid is ceil(n_rv / 32) * ceil(G / 8) * nb workgroups (launch_downcast).
   int64_t n_rv = (nr + NV - 1) / NV;
-  int64_t blocks_r = (n_rv + 255) / 256;
+  int64_t blocks_r = (n_rv + 31) / 32;
+  int64_t g_chunks = (G + 7) / 8;
   int64_t bid = blockIdx.x;
   int64_t br = bid % blocks_r;
   int64_t t = bid / blocks_r;
-  int64_t g = t % G;
-  int64_t b = t / G;
-  int64_t rv = br * 256 + threadIdx.x;
-  if (rv >= n_rv) return;
+  int64_t g = (t % g_chunks) * 8 + threadIdx.x % 8;
+  int64_t b = t / g_chunks;
+  int64_t rv = br * 32 + threadIdx.x / 8;
+  if (rv >= n_rv || g >= G || b >= nb) return;
   int64_t r0 = rv * NV;
   constexpr int ES = DT == TAMD_F32 ? 4 : 2;
   const char *base = (const char *)src + (b * ssb + g * 32 * ssl + r0) * ES;
@@ -335,12 +339,12 @@ int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t 
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(src, 16) && (ssb * ES) % 16 == 0 && (ssl * ES) % 16 == 0;
   if (vec) {
-    int64_t blocks = ((nr / NV + 255) / 256) * G * nb;
+    int64_t blocks = ((nr / NV + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
     downcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
                                                                         scales, csb, csr, mode);
   } else {
-    int64_t blocks = ((nr + 255) / 256) * G * nb;
+    int64_t blocks = ((nr + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
     downcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
                                                                        scales, csb, csr, mode);
