@@ -158,3 +158,24 @@ def test_mxfp8_quant_dequant_exact(vdt, max_q, dst, device):
     w = torch.nn.functional.pad(w, (0, 0, 0, 16)).to(device)
     q, s = downcast_to_mxfp(w, vdt, axis=1)
     assert torch.equal(upcast_from_mxfp(q, s, dst, axis=1), w)
+
+
+@pytest.mark.parametrize("anchor", [6.0, 4.0, 1.0, 448.0, 3.0e38])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_every_bf16_value_against_oracle(anchor, axis, device):
+    """All 65536 bfloat16 bit patterns (NaNs and infinities included), 31 to a group next to an anchor that fixes the
+    group's scale: codes and scales must equal the oracle's for each of them, along a contiguous and a strided axis."""
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    finite = allv[torch.isfinite(allv.float()) & (allv.float().abs() <= anchor)]
+    pad = (-finite.numel()) % 31
+    vals = torch.cat([finite, torch.zeros(pad, dtype=torch.bfloat16)]).view(-1, 31)
+    x = torch.cat([torch.full((vals.shape[0], 1), anchor, dtype=torch.bfloat16), vals], dim=1)  # [groups, 32]
+    if axis == 0:
+        x = x.t().contiguous()  # [32, groups]: quantised axis strided
+    for vdt in (torch.uint8, torch.float8_e4m3fn, torch.float8_e5m2):
+        if vdt != torch.uint8 and axis == 0:
+            continue
+        rv, rs = downcast_to_mxfp_ref(x, vdt, axis)
+        v, s = downcast_to_mxfp(x.to(device), vdt, axis)
+        assert torch.equal(s.cpu(), rs)
+        assert torch.equal(v.cpu().view(torch.uint8), rv.view(torch.uint8))
