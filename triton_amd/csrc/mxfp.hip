@@ -19,6 +19,16 @@ TAMD_DEVICE uint32_t e2m1_code(float q) {
   return c | ((f32_to_bits(q) >> 28) & 8u);
 }
 
+// Two e2m1 codes (q0 in the low nibble) by the hardware conversion: round to nearest even onto the e2m1 grid,
+// saturating at 6 (v_cvt_scalef32_pk_fp4_f32 with a unit scale).  NaN has no e2m1 code: like e2m1_code it becomes
+// the largest magnitude with the sign of the NaN's pattern.
+TAMD_DEVICE uint32_t e2m1_pair(float q0, float q1) {
+  uint32_t c = (uint32_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, q0, q1, 1.0f, 0) & 0xFFu;
+  if (q0 != q0) c = (c & 0xF0u) | 7u | ((f32_to_bits(q0) >> 28) & 8u);
+  if (q1 != q1) c = (c & 0x0Fu) | ((7u | ((f32_to_bits(q1) >> 28) & 8u)) << 4);
+  return c;
+}
+
 // Value kinds of a microscaled tensor: e2m1 codes (two per byte), or fp8 bytes.  Largest magnitude and
 // largest power of two of each (mxfp.py:206-209, mxfp_details/_downcast_to_mxfp.py:24-31).
 constexpr int QK_E2M1 = 0, QK_E4M3 = 1, QK_E5M2 = 2;
@@ -129,7 +139,7 @@ __global__ __launch_bounds__(256) void downcast_rows_kernel(
   if constexpr (QK == QK_E2M1) {
     uint32_t packed = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) packed |= e2m1_code(v[j] * qs) << (4 * j);
+    for (int j = 0; j < 8; j += 2) packed |= e2m1_pair(v[j] * qs, v[j + 1] * qs) << (4 * j);
     if (!live) return;
     *(uint32_t *)(vals + b * vsb + r * vsr + g * 16 + sub * 4) = packed;
   } else {
@@ -184,7 +194,7 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
     float qs = group_scale(mx[0], mode, sbyte);
     uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int l = 0; l < 32; ++l) w[l >> 3] |= e2m1_code(v[l] * qs) << (4 * (l & 7));
+    for (int l = 0; l < 32; l += 2) w[l >> 3] |= e2m1_pair(v[l] * qs, v[l + 1] * qs) << (4 * (l & 7));
     *(uint4 *)(vals + b * vsb + r0 * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
     scales[b * csb + r0 * csr + g] = (uint8_t)sbyte;
   } else {
@@ -209,7 +219,7 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
       float qs = group_scale(mx[c], mode, sbyte);
       uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int l = 0; l < 32; ++l) w[l >> 3] |= e2m1_code(elem(l, c) * qs) << (4 * (l & 7));
+      for (int l = 0; l < 32; l += 2) w[l >> 3] |= e2m1_pair(elem(l, c) * qs, elem(l + 1, c) * qs) << (4 * (l & 7));
       *(uint4 *)(vals + b * vsb + (r0 + c) * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
       scales[b * csb + (r0 + c) * csr + g] = (uint8_t)sbyte;
     }
