@@ -9,19 +9,9 @@
 
 namespace tamd {
 
-// e2m1 code (sign in bit 3) of q: nearest grid value, ties to the even code.
-TAMD_DEVICE uint32_t e2m1_code(float q) {
-  float a = __builtin_fabsf(q);
-  uint32_t c = (uint32_t)(a > 0.25f) + (uint32_t)(a >= 0.75f) + (uint32_t)(a > 1.25f) +
-               (uint32_t)(a >= 1.75f) + (uint32_t)(a > 2.5f) + (uint32_t)(a >= 3.5f) +
-               (uint32_t)(a > 5.0f);
-  if (a != a) c = 7u;
-  return c | ((f32_to_bits(q) >> 28) & 8u);
-}
-
 // Two e2m1 codes (q0 in the low nibble) by the hardware conversion: round to nearest even onto the e2m1 grid,
-// saturating at 6 (v_cvt_scalef32_pk_fp4_f32 with a unit scale).  NaN has no e2m1 code: like e2m1_code it becomes
-// the largest magnitude with the sign of the NaN's pattern.
+// saturating at 6 (v_cvt_scalef32_pk_fp4_f32 with a unit scale).  NaN has no e2m1 code: it becomes the largest
+// magnitude with the sign bit of the NaN's pattern.
 TAMD_DEVICE uint32_t e2m1_pair(float q0, float q1) {
   uint32_t c = (uint32_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, q0, q1, 1.0f, 0) & 0xFFu;
   if (q0 != q0) c = (c & 0xF0u) | 7u | ((f32_to_bits(q0) >> 28) & 8u);
