@@ -93,6 +93,25 @@ def test_host_only_entry_points(lib):
     assert lib.tamd_bitmatrix_metadata_workspace(0, 128) >= 0
 
 
+def test_matmul_rejects_degenerate_problems_before_any_launch(lib):
+    """Argument checks that return before the first HIP call (so they run without a device): a null argument block,
+    negative sizes, and K == 0 with non-null pointers, which the kernels' K loops are not built for."""
+    from triton_amd import _lib
+    assert lib.tamd_matmul(None, None) == _lib.E_INVALID
+    a = _lib.MatmulArgs()
+    a.x, a.w, a.y, a.w_mx_scale = 0x1000, 0x2000, 0x3000, 0x4000  # never dereferenced on these paths
+    a.x_dtype, a.w_dtype, a.y_dtype = _lib.BF16, _lib.MXFP4, _lib.BF16
+    a.M, a.N, a.K, a.n_experts = 16, 256, 0, 1
+    a.x_stride_m, a.w_stride_k, a.w_stride_n, a.w_mx_stride_k, a.w_mx_stride_n, a.y_stride_m = 0, 1, 0, 1, 0, 256
+    assert lib.tamd_matmul(C.byref(a), None) == _lib.E_UNSUPPORTED
+    a.K = -32
+    assert lib.tamd_matmul(C.byref(a), None) == _lib.E_INVALID
+    a.K, a.n_experts = 64, 0
+    assert lib.tamd_matmul(C.byref(a), None) == _lib.E_INVALID
+    a.n_experts, a.K = 1, 48  # not a whole number of 32-element scale groups
+    assert lib.tamd_matmul(C.byref(a), None) == _lib.E_INVALID
+
+
 def test_no_cpu_fallback_in_product():
     """The package never imports the oracle and refuses CPU tensors."""
     import torch

@@ -163,8 +163,9 @@ def test_mxfp8_quant_dequant_exact(vdt, max_q, dst, device):
 @pytest.mark.parametrize("anchor", [6.0, 4.0, 1.0, 448.0, 3.0e38])
 @pytest.mark.parametrize("axis", [0, 1])
 def test_every_bf16_value_against_oracle(anchor, axis, device):
-    """All 65536 bfloat16 bit patterns (NaNs and infinities included), 31 to a group next to an anchor that fixes the
-    group's scale: codes and scales must equal the oracle's for each of them, along a contiguous and a strided axis."""
+    """Every finite bfloat16 bit pattern up to the anchor, 31 to a group next to an anchor that fixes the group's
+    scale: codes and scales must equal the oracle's for each of them, along a contiguous and a strided axis.
+    (Non-finite inputs are outside the contract: the reference's own twins disagree on them.)"""
     allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
     finite = allv[torch.isfinite(allv.float()) & (allv.float().abs() <= anchor)]
     pad = (-finite.numel()) % 31
@@ -179,3 +180,100 @@ def test_every_bf16_value_against_oracle(anchor, axis, device):
         v, s = downcast_to_mxfp(x.to(device), vdt, axis)
         assert torch.equal(s.cpu(), rs)
         assert torch.equal(v.cpu().view(torch.uint8), rv.view(torch.uint8))
+
+
+# ---------------------------------------------------------------------------- the e2m1 rounding of float32 / float16 sources
+# The kernels round with the hardware conversion (v_cvt_scalef32_pk_fp4_f32); the reference's bit path (restated in
+# oracle/mxfp_ref.py:e2m1_codes_from_f32 and pinned on the CPU by an exact-rational brute force) is round to nearest,
+# ties to even.  The cases below are the ones where the two could part: values one ulp either side of every
+# midpoint of the e2m1 grid, at every scale a float32 group can have, tiny and subnormal inputs, signed zeros.
+
+E2M1_MIDPOINTS = (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0)
+
+
+def _check_against_oracle(x, axis, device, vdt=torch.uint8):
+    rv, rs = downcast_to_mxfp_ref(x, vdt, axis)
+    v, s = downcast_to_mxfp(x.to(device), vdt, axis)
+    assert torch.equal(s.cpu(), rs), "scales differ"
+    bad = (v.cpu().view(torch.uint8) != rv.contiguous().view(torch.uint8)).nonzero()
+    assert bad.numel() == 0, f"{bad.shape[0]} bytes differ, first at {bad[0].tolist()}"
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_f32_tie_neighbours_at_every_scale(axis, device):
+    """Anchor 6 * 2^e fixes the scale 2^e of a group; its other members are (midpoint -1 ulp, midpoint, midpoint +1 ulp)
+    * 2^e of either sign for all seven midpoints, for every e at which they are normal float32 numbers."""
+    mids = torch.tensor(E2M1_MIDPOINTS, dtype=torch.float32)
+    bits = mids.view(torch.int32)
+    cand = torch.stack([(bits - 1).view(torch.float32), mids, (bits + 1).view(torch.float32)], dim=1).reshape(-1)  # 21
+    cand = torch.cat([cand, -cand])  # 42 values, exact multiples of 2^-25
+    groups = []
+    for e in range(-122, 125):
+        sc = torch.tensor(2.0, dtype=torch.float64)**e
+        vals = (cand.double() * sc).float()
+        assert torch.equal(vals.double(), cand.double() * sc)  # scaling by a power of two is exact here
+        for part in (vals[:21], vals[21:]):
+            g = torch.zeros(32, dtype=torch.float32)
+            g[0] = float(6.0 * sc)
+            g[1:22] = part
+            groups.append(g)
+    x = torch.stack(groups)  # [groups, 32]
+    if axis == 0:
+        x = x.t().contiguous()
+    _check_against_oracle(x, axis, device)
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_f32_tiny_subnormal_and_signed_zero_inputs(axis, device):
+    """Members far below the group's scale round to a zero that keeps its sign (the reference's bit path carries the
+    sign bit through); subnormal inputs and whole groups of subnormals (scale byte 0 or 1) included."""
+    tiny = torch.tensor([0.0, -0.0, 1e-45, -1e-45, 1e-40, -1e-40, 1.17549435e-38, -1.17549435e-38, 1e-30, -1e-30, 0.24999999, -0.24999999,
+                         0.25, -0.25, 0.25000003, -0.25000003], dtype=torch.float32)
+    groups = []
+    for anchor in (1.0, 6.0, 5.9999995, 1e-30, 1.17549435e-38, 3e-39, 1e-44, 0.0, 3.0e38):
+        g = torch.zeros(32, dtype=torch.float32)
+        g[0] = anchor
+        g[1:17] = tiny if anchor >= 1e-30 else tiny * 0 + torch.tensor([0.0, -0.0, 1e-45, -1e-45] * 4, dtype=torch.float32)
+        g[17:] = torch.tensor([anchor * f for f in (-1.0, 0.5, -0.5, 0.75, -0.75, 0.3, -0.3, 0.2, -0.2, 0.1, -0.1, 0.04, -0.04, 0.9, -0.9)],
+                              dtype=torch.float32)
+        groups.append(g)
+    x = torch.stack(groups)
+    if axis == 0:
+        x = x.t().contiguous()
+    _check_against_oracle(x, axis, device)
+
+
+def test_f32_random_bit_patterns(device):
+    """2^24 random finite float32 bit patterns (every exponent, so most members vanish against their group's maximum)
+    and 2^22 values whose exponents stay within six binades of their group's anchor (so most members land on the
+    grid proper), against the oracle."""
+    g = torch.Generator().manual_seed(7)
+    bits = torch.randint(-2**31, 2**31, (2**24, ), generator=g, dtype=torch.int64).to(torch.int32)
+    x = bits.view(torch.float32)
+    x = torch.where(torch.isfinite(x), x, torch.zeros_like(x)).view(-1, 4096)
+    _check_against_oracle(x, 1, device)
+    n = 2**22
+    mant = torch.randint(0, 2**23, (n, ), generator=g, dtype=torch.int64)
+    sign = torch.randint(0, 2, (n, ), generator=g, dtype=torch.int64) << 31
+    base = torch.randint(8, 250, (n // 32, 1), generator=g, dtype=torch.int64)
+    expo = (base - torch.randint(0, 7, (n // 32, 32), generator=g, dtype=torch.int64)).reshape(-1)
+    y = (sign | (expo << 23) | mant).to(torch.int32).view(torch.float32).view(-1, 2048)
+    _check_against_oracle(y, 1, device)
+    _check_against_oracle(y[:4096].t().contiguous(), 0, device)  # the same values along a strided axis
+
+
+@pytest.mark.parametrize("anchor", [6.0, 4.0, 1.0, 448.0, 65504.0, 6.1e-5, 6e-8])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_every_f16_value_against_oracle(anchor, axis, device):
+    """Every finite float16 bit pattern (subnormals included) up to the anchor, as in the bfloat16 test above."""
+    allv = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    finite = allv[torch.isfinite(allv.float()) & (allv.float().abs() <= anchor)]
+    pad = (-finite.numel()) % 31
+    vals = torch.cat([finite, torch.zeros(pad, dtype=torch.float16)]).view(-1, 31)
+    x = torch.cat([torch.full((vals.shape[0], 1), anchor, dtype=torch.float16), vals], dim=1)
+    if axis == 0:
+        x = x.t().contiguous()
+    for vdt in (torch.uint8, torch.float8_e4m3fn, torch.float8_e5m2):
+        if vdt != torch.uint8 and axis == 0:
+            continue
+        _check_against_oracle(x, axis, device, vdt)

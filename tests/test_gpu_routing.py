@@ -53,6 +53,33 @@ def test_topk_n_rows_and_provided_indx(device):
     assert torch.equal(sp.mask.storage.data.cpu().view(torch.int32), bits)
 
 
+@pytest.mark.parametrize("n_rows,n_rows_max", [(70, 100), (0, 33), (4097, 5000)])
+def test_topk_n_rows_bounds_the_metadata(n_rows, n_rows_max, device):
+    """Rows at and beyond `n_rows` are not routed: whatever their index entries hold (here: valid-looking expert
+    ids), the histogram and the ordering count the first n_rows rows only and pad with -1
+    (tensor_details/bitmatrix.py:138-145 of the reference bounds both stages by bitmatrix.shape[0])."""
+    torch.manual_seed(4)
+    k, n_cols = 4, 64
+    x = torch.randn(n_rows_max, n_cols)
+    y_indx = torch.full((n_rows_max, k), 7, dtype=torch.int16, device=device)  # poison: the kernel leaves the tail alone
+    vals, indx, bits = R.topk_ref(x, k, n_rows=n_rows)
+    y_indx[:n_rows] = indx[:n_rows].to(torch.int16).to(device)
+    sp = topk(x.to(device), k, y_indx=y_indx, n_rows=n_rows)
+    assert sp.mask.shape[0] == n_rows
+    assert torch.equal(sp.indx[n_rows:].cpu(), torch.full((n_rows_max - n_rows, k), 7, dtype=torch.int16))
+    ref = R.bitmatrix_metadata_ref(indx[:n_rows], n_cols)
+    pad = torch.full(((n_rows_max - n_rows) * k, ), -1, dtype=torch.int32)
+    m = sp.mask_metadata
+    assert torch.equal(m.col_sum.cpu(), ref.col_sum)
+    assert torch.equal(m.col_sorted_indx.cpu(), torch.cat([ref.col_sorted_indx, pad]))
+    assert torch.equal(m.row_sorted_indx.cpu(), torch.cat([ref.row_sorted_indx, pad]))
+    # without provided indices the tail of indx is whatever the allocation held; the metadata must not depend on it
+    sp2 = topk(x.to(device), k, n_rows=n_rows)
+    assert torch.equal(sp2.mask_metadata.col_sum.cpu(), ref.col_sum)
+    assert torch.equal(sp2.mask_metadata.col_sorted_indx.cpu(), torch.cat([ref.col_sorted_indx, pad]))
+    assert torch.equal(sp2.mask_metadata.row_sorted_indx.cpu(), torch.cat([ref.row_sorted_indx, pad]))
+
+
 @pytest.mark.parametrize("n_rows", [7, 256, 17111])
 @pytest.mark.parametrize("n_cols", [13, 32, 128, 811])
 @pytest.mark.parametrize("k", [1, 4, 8])

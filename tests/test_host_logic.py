@@ -102,6 +102,32 @@ def test_opt_flags_constraints_scope_and_errors():
     assert OF.make_opt_flags(16384, 5760, 2880, 128, True).block_m == 128
 
 
+def test_opt_flags_constraint_keys_are_validated():
+    """Unknown keys are a caller's mistake (AssertionError, matmul_details/opt_flags.py:71-73 of the reference); known
+    keys must hold for the flags that come out (:46-50), so values the fixed tile cannot honour raise instead of
+    being dropped."""
+    OF.reset_opt_flags_constraints()
+    with OF.scoped_opt_flags_constraints({"blok_m": 64}):
+        with pytest.raises(AssertionError, match="unsupported constraint"):
+            OF.make_opt_flags(100, 64, 64, 1, False)
+    for key, bad, good in (("block_n", 128, 256), ("block_k", 64, 128), ("num_warps", 8, 4), ("epilogue_subtile", 2, 1),
+                           ("idle_sms", 4, 0)):
+        with OF.scoped_opt_flags_constraints({key: bad}):
+            with pytest.raises(OF.InapplicableConstraint, match=key):
+                OF.make_opt_flags(100, 64, 64, 1, False)
+        with OF.scoped_opt_flags_constraints({key: good}):
+            flags = OF.make_opt_flags(100, 64, 64, 1, False)
+            assert getattr(flags, key, good) == good
+        with OF.scoped_opt_flags_constraints({key: None}):
+            OF.make_opt_flags(100, 64, 64, 1, False)
+    with OF.scoped_opt_flags_constraints({"disable_mx4_block_swap": True, "is_persistent": False}):
+        OF.make_opt_flags(100, 64, 64, 1, False)
+    # max_allowable_mn switches a requested split_k off once the output is large (opt_flags.py:37-43, 114-117)
+    with OF.scoped_opt_flags_constraints({"split_k": 4, "max_allowable_mn": 100 * 64}):
+        assert OF.make_opt_flags(100, 64, 4096, 1, False).split_k == 1
+        assert OF.make_opt_flags(99, 64, 4096, 1, False).split_k == 4
+
+
 def test_opt_flags_constraints_are_per_thread():
     OF.reset_opt_flags_constraints()
     seen = {}

@@ -20,6 +20,8 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
   if (a.M < 0 || a.N < 0 || a.K < 0 || a.n_experts < 1) return TAMD_E_INVALID;
   if (a.n_experts == 1) a.w_stride_e = a.w_mx_stride_e = a.bias_stride_e = 0;  // never used; keeps the alignment checks honest
   if (a.M == 0 || a.N == 0) return 0;
+  // K == 0 would be a bias-only problem; no kernel is built for it, and the K loops assume at least one stage
+  if (a.K == 0) return TAMD_E_UNSUPPORTED;
   if (!a.x || !a.w || !a.y) return TAMD_E_INVALID;
   if (a.activation != TAMD_ACT_NONE && a.activation != TAMD_ACT_SWIGLU) return TAMD_E_INVALID;
   if (a.activation == TAMD_ACT_SWIGLU && (a.N % 2) != 0) return TAMD_E_INVALID;

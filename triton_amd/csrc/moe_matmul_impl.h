@@ -113,7 +113,15 @@ template <int BLOCK_M, int EXTRA>
 TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid_total, int group_m, Tile &t) {
   // XCD-aware remap: hardware deals workgroups round-robin to the 8 XCDs; give each XCD a
   // contiguous range of tiles so neighbours (same expert, adjacent columns) share one L2.
+  // A ragged launch is sized for the worst split of the rows over the experts (grid_total), about twice what a
+  // balanced routing needs; the schedule's real entries come first and their number is block_offs[n_experts].  The
+  // XCD ranges are cut from that number, read here, so that all eight XCDs share the real tiles; the rest exit.
+  if (a.block_schedule && a.block_offs) {
+    const int64_t real_total = (int64_t)a.block_offs[a.n_experts] * grid_n;
+    grid_total = real_total < grid_total ? real_total : grid_total;
+  }
   const int64_t per_xcd = (grid_total + 7) / 8;
+  if ((int64_t)(blockIdx.x / 8) >= per_xcd) return false;
   int64_t pid = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (pid >= grid_total) return false;
   // Tiles are walked in groups of `group_m` row blocks: row block fastest inside a group, then the
@@ -468,6 +476,9 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const int wave = tid / kWave, lane = tid % kWave;
   const int c32 = lane % 32, h = lane / 32;
   const int K = a.K, N = a.N, G = K / 32;
+  // a wave whose 64 columns lie beyond N (last column tile) copies its share of the activations and keeps the
+  // barriers, but neither fetches weights nor runs MFMAs
+  const bool wave_live = t.n0 + wave * 64 < N;
 
   const v4i_t rx = make_rsrc((const uint8_t *)a.x + (int64_t)t.z * a.x_stride_z * ESZ, kOob);
   const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
@@ -567,10 +578,12 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   uint32_t a_off[NFR];
 #pragma unroll
   for (int i = 0; i < NFR; ++i) {
-    int r = i * 32 + a_rin;
-    int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
-    uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
-    a_off[i] = src * (uint32_t)(a.x_stride_m * ESZ) + a_chunk * 16;
+    const int r = i * 32 + a_rin;
+    // rows past the end of the slice are never stored: they are copied as zeros (out-of-range offset), which
+    // keeps the matrix cores' inputs quiet for the padding of a ragged tile
+    const int rr = t.off_m + (r < t.rows ? r : t.rows - 1);
+    const uint32_t src = a.gather_indx ? (uint32_t)a.gather_indx[t.start_m + rr] : (uint32_t)(t.start_m + rr);
+    a_off[i] = r < t.rows ? src * (uint32_t)(a.x_stride_m * ESZ) + a_chunk * 16 : kOob;
   }
   // ---- weight DMA: instruction j copies LDS positions j*16 + lane/4, part slot lane%4
   uint32_t w_off[4];
@@ -608,7 +621,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     const int kb = sup * KB;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t bkill = kb + w_part[j] * 32 < K ? 0u : kOob;
+      const uint32_t bkill = (wave_live && kb + w_part[j] * 32 < K) ? 0u : kOob;
       dma16(rw, lds_b + j * 1024, w_off[j] | bkill, kb >> 1);
     }
   };
@@ -642,6 +655,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 
   auto compute = [&](int it, auto qc) {
     constexpr int q = decltype(qc)::value;
+    if (!wave_live) return;
     const uint8_t *buf = lds + (it & 1) * A_STAGE;
     if constexpr (FP8) {
       // one stage = 128 K = two scaled MFMAs per (row fragment, column fragment)

@@ -119,8 +119,15 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         c_mx_scale = _data(c_mx_scale)
         if c_mx_scale.dtype != torch.uint8 or (precision_config.c_microblock_size or MXFP_BLOCK_SIZE) != MXFP_BLOCK_SIZE:
             raise NotImplementedError("output scales are built as e8m0 bytes per 32 columns")
-        precision_config.c_microblock_size = MXFP_BLOCK_SIZE
-        precision_config.c_value_pack_factor = 1
+        if precision_config.c_value_pack_factor != 1:
+            raise NotImplementedError("packed output values (c_value_pack_factor != 1) are not built")
+        if precision_config.c_microblock_size is None:
+            precision_config.c_microblock_size = MXFP_BLOCK_SIZE  # filled in for the caller, as matmul.py:362-363 does
+    # fields that change the result and have no kernel here must not be dropped silently
+    if precision_config.a_mx_tensor_scale is not None or precision_config.b_mx_tensor_scale is not None:
+        raise NotImplementedError("per-tensor scales on top of microscales (NVFP4-style) are not built")
+    if precision_config.acc_scale != 1.0:
+        raise NotImplementedError("acc_scale other than 1.0 is not built")
     a_mx_scale = precision_config.a_mx_scale
     if a_mx_scale is not None:
         a_mx_scale = _data(a_mx_scale)

@@ -72,22 +72,46 @@ def scoped_opt_flags(opt_flags: OptFlags):
         _opt_flags.reset(token)
 
 
+# keys the reference accepts on this target (matmul_details/opt_flags.py:71-73); any other key is a caller's mistake
+CONSTRAINTS_SUPPORTED = frozenset({"block_m", "block_n", "block_k", "split_k", "is_persistent", "epilogue_subtile",
+                                   "idle_sms", "max_allowable_mn", "num_warps", "disable_mx4_block_swap"})
+
+
+def max_allowable_mn(max_mn: int, m: int, n: int, split_k: int) -> int:
+    """split_k only while the output is small (matmul_details/opt_flags.py:37-43)."""
+    return 1 if m * n >= max_mn else split_k
+
+
 def make_opt_flags(m: int, n: int, k: int, n_slices: int, ragged: bool,
                    expected_slice_size: Optional[int] = None) -> OptFlags:
     """Picks BLOCK_M from the expected rows per slice (no device read): the smallest
     tile that covers them, capped at 128, so that ragged slices waste at most one
-    partly filled 16-row fragment per block."""
+    partly filled 16-row fragment per block.
+
+    Constraints are validated as the reference validates them (opt_flags.py:71-73, 46-50): an unknown key is
+    an AssertionError; a known key has to hold for the flags that come out, and since the tile's width, depth
+    and wave count are fixed in the kernels (256 columns, 128 K, 4 waves, no persistent kernel, no epilogue
+    sub-tiling, no idle CUs) any other value for them raises InapplicableConstraint instead of being dropped."""
     forced = _opt_flags.get()
     if forced is not None:
         return forced
     c = _constraints()
-    for key in ("is_persistent", ):
-        if c.get(key):
-            raise InapplicableConstraint("there is no persistent kernel on gfx950")
+    unsupported = set(c) - CONSTRAINTS_SUPPORTED
+    assert not unsupported, f"Given unsupported constraint: {unsupported}"
+    if c.get("is_persistent"):
+        raise InapplicableConstraint("there is no persistent kernel on gfx950")
+    fixed = OptFlags(block_m=0)
+    for key, have in (("block_n", fixed.block_n), ("block_k", fixed.block_k), ("num_warps", fixed.num_warps),
+                      ("epilogue_subtile", 1), ("idle_sms", 0)):
+        want = c.get(key)
+        if want is not None and int(want) != have:
+            raise InapplicableConstraint(f"{key} is fixed at {have} in the gfx950 kernels (asked for {want})")
     split_k = c.get("split_k")
     split_k = 1 if split_k is None else int(split_k)
     if split_k < 1:
         raise InapplicableConstraint("split_k must be positive")
+    if (c.get("max_allowable_mn") or 0) > 0 and c.get("split_k") is not None:
+        split_k = max_allowable_mn(int(c["max_allowable_mn"]), m, n, split_k)
     rows = m
     if ragged:
         rows = expected_slice_size if expected_slice_size is not None else max(1, m // max(1, n_slices))
