@@ -32,6 +32,7 @@ extern "C" {
 #define TAMD_E_INVALID (-1)     /* bad shape / stride / pointer / enum */
 #define TAMD_E_UNSUPPORTED (-2) /* valid in the reference, not built here */
 #define TAMD_E_ALIGNMENT (-3)   /* pointer or stride not aligned as the kernel needs */
+#define TAMD_E_TOO_LARGE (-4)   /* problem exceeds a fixed capacity of the entry point (see its comment) */
 
 /* element types */
 #define TAMD_F32 0
@@ -142,6 +143,23 @@ int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, i
                           int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
                           int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
                           int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream);
+
+/*
+ * tamd_routing_metadata for callers that cannot allocate (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, where every workspace is a torch allocation
+ * made per call.  Same arguments and results as tamd_routing_metadata without `workspace`: the intermediate
+ * tables live in a fixed 4 MiB array inside the library's code object (one copy per GPU, held until the process
+ * ends).  Calls no allocating routine.  Problems whose workspace
+ * (tamd_bitmatrix_metadata_workspace(n_indx, n_cols) int32 elements) exceeds
+ * tamd_routing_metadata_static_max_workspace() elements return TAMD_E_TOO_LARGE and launch nothing.  All calls on
+ * one GPU share that array: calls that overlap in time on the same GPU (different streams or threads) race; calls
+ * on one stream are ordered and safe.
+ */
+int64_t tamd_routing_metadata_static_max_workspace(void);
+int tamd_routing_metadata_static(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
+                                 int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                 int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
+                                 int64_t sched_pitch, int max_n_blocks, void *stream);
 
 /* activation fused into the matmul epilogue (matmul.py:40-43, swiglu_details/_swiglu.py:55-70) */
 #define TAMD_ACT_NONE 0

@@ -16,7 +16,7 @@ LIB_PATH = os.environ.get("TAMD_LIB") or os.path.join(_HERE, "libtriton_amd.so")
 F32, F16, BF16, FP8_E4M3, FP8_E5M2, MXFP4 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_SWIGLU = 0, 1
 SCALE_STRIDED, SCALE_CDNA4 = 0, 1
-E_INVALID, E_UNSUPPORTED, E_ALIGNMENT = -1, -2, -3
+E_INVALID, E_UNSUPPORTED, E_ALIGNMENT, E_TOO_LARGE = -1, -2, -3, -4
 
 _TORCH_CODE = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16,
@@ -72,6 +72,9 @@ _SIGNATURES = {
     "tamd_ragged_metadata": ([_PTR, _INT, _PTR, _I64, _PTR, _I64, _INT, _PTR], C.c_int),
     "tamd_routing_metadata": ([_PTR, _INT, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _I64, _INT,
                                _PTR, _PTR], C.c_int),
+    "tamd_routing_metadata_static_max_workspace": ([], C.c_int64),
+    "tamd_routing_metadata_static": ([_PTR, _INT, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _I64,
+                                      _INT, _PTR], C.c_int),
     "tamd_matmul": ([C.POINTER(MatmulArgs), _PTR], C.c_int),
     "tamd_reduce": ([_PTR, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _PTR, _I64, _I64, _I64, _PTR, _I64, _I64, _I64,
                      _PTR, _INT, _I64, _I64, _PTR], C.c_int),
@@ -105,7 +108,7 @@ def check(rc: int, what: str):
     msg = f"{what}: {lib().tamd_error_string(rc).decode()} (code {rc})"
     if rc == E_UNSUPPORTED:
         raise NotImplementedError(msg)
-    if rc in (E_INVALID, E_ALIGNMENT):
+    if rc in (E_INVALID, E_ALIGNMENT, E_TOO_LARGE):
         raise ValueError(msg)
     raise RuntimeError(msg)
 

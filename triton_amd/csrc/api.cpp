@@ -9,6 +9,7 @@ extern "C" const char *tamd_error_string(int code) {
     case TAMD_E_INVALID: return "invalid argument";
     case TAMD_E_UNSUPPORTED: return "combination not supported by this build";
     case TAMD_E_ALIGNMENT: return "pointer or stride misaligned";
+    case TAMD_E_TOO_LARGE: return "problem exceeds the fixed capacity of this entry point";
     default: return code > 0 ? "HIP runtime error" : "unknown error";
   }
 }

@@ -2,9 +2,16 @@
 // stable expert-major ordering of the (token, slot) pairs, and the ragged-tensor
 // block metadata.  Integer work only; wave64 ballots / shuffles, no float atomics,
 // results independent of scheduling.
+#include <atomic>
+
 #include "common.h"
 
 namespace tamd {
+
+// Workspace of tamd_routing_metadata_static: lives in the code object instead of an allocation.  Every GPU that
+// loads the library holds its own copy (4 MiB) until the process ends.
+constexpr int64_t kStaticWorkspaceInts = 1 << 20;
+static __device__ __align__(256) int32_t scratch[kStaticWorkspaceInts];
 
 // ---------------------------------------------------------------------------
 // top-k
@@ -627,10 +634,10 @@ bool ragged_between(void *p) {
 }
 }  // namespace
 
-extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
-                                     int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
-                                     int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
-                                     int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream) {
+static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
+                                 int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                 int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
+                                 int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream) {
   if (n_indx < 0 || n_cols <= 0 || n_cols > 16384 || n_indx > 0x7FFFFFFF || k < 1) return TAMD_E_INVALID;
   if (max_n_blocks < 0 || offs_pitch < n_cols + 1 || sched_pitch < max_n_blocks) return TAMD_E_INVALID;
   if (!col_sum || !workspace || !offs || (max_n_blocks > 0 && !schedule)) return TAMD_E_INVALID;
@@ -674,4 +681,50 @@ extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_
   RaggedCtx ctx{col_sum, n_cols, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, (hipStream_t)stream};
   return launch_bitmatrix_metadata(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx,
                                    row_sorted_indx, gather_indx, workspace, (hipStream_t)stream, ragged_between, &ctx);
+}
+
+extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
+                                     int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                     int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
+                                     int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream) {
+  return routing_metadata_impl(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx, row_sorted_indx,
+                               gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, workspace, stream);
+}
+
+// Device address of `scratch` on the current device.  In host code the array's name only stands for the symbol: its
+// memory is reached through the address the runtime reports, which differs from GPU to GPU and is looked up once
+// per device (with that device current) and kept.
+static int static_workspace(int32_t **out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int32_t *> ptr_of_device[kMaxDevices];
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return TAMD_E_UNSUPPORTED;
+  int32_t *p = ptr_of_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return TAMD_E_INVALID;
+    ptr_of_device[dev].store(p, std::memory_order_release);  // two racing first calls store the same address
+  }
+  *out = p;
+  return 0;
+}
+
+extern "C" int64_t tamd_routing_metadata_static_max_workspace(void) { return kStaticWorkspaceInts; }
+
+extern "C" int tamd_routing_metadata_static(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
+                                            int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
+                                            int32_t *gather_indx, int32_t *offs, int64_t offs_pitch,
+                                            int32_t *schedule, int64_t sched_pitch, int max_n_blocks, void *stream) {
+  if (n_indx < 0 || n_cols <= 0) return TAMD_E_INVALID;
+  if (make_meta_plan(n_indx, n_cols).total > kStaticWorkspaceInts) return TAMD_E_TOO_LARGE;
+  int32_t *ws = nullptr;
+  const int rc = static_workspace(&ws);
+  if (rc != 0) return rc;
+  // every entry of the workspace that a launch reads is written earlier by the same call (per-chunk prefixes and
+  // per-workgroup totals by the histogram kernel, the prefix tables by the scan kernel): nothing has to start at zero
+  return routing_metadata_impl(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx, row_sorted_indx,
+                               gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, ws, stream);
 }
