@@ -1,15 +1,20 @@
 """Benchmark of the quantized-MoE hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload fc1_prefill|fc1_decode|dense|routing]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-configs]
 
 Default workload: MoE up-projection + fused SwiGLU at the prefill shape (T=4096 tokens, hidden 2880,
 128 experts, top-4, MXFP4 weights [128, 2880, 5760], bf16 activations).  A step is one pass of the path over
 one batch: routing(logits) then matmul_ogs(gather -> grouped GEMM -> bias + SwiGLU).  Inputs (logits,
-activations, quantised weights) are resident in HBM before the timed region.  Prints ONE JSON line.
+activations, quantised weights) are resident in HBM before the timed region.  Prints ONE JSON line; with the
+default workload the line also carries short runs of every other configuration of the path ("configs": dense
+product, routing, decode, fp8 down projection + combine, quantise, dequantise), each with its kernel time,
+achieved rate, roofline fraction and parity flags.
 """
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 
@@ -22,10 +27,6 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_MXFP4_TFLOPS = 10100.0
-
-# HBM bytes per launch of the dominant kernel (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00 KiB from rocprofv3 --pmc,
-# factors from the hbm_copy workload).  Counters cannot be read from inside this process; re-measure after kernel changes.
-MEASURED_TRAFFIC = {"fc1_prefill": 1611457371, "fc1_decode": 976176743, "fc2_combine": 1497319402}
 
 WORKLOADS = {
     # name: (T, E, k, K, N, swiglu)
@@ -42,10 +43,91 @@ WORKLOADS = {
     "fc2_decode": dict(T=64, E=128, k=4, K=2880, N=2880, act=False, fc2=True),
     # BASELINE config 1: one dense bf16 x MXFP4 product with bias (launch / latency bound: 7.6 MB, 4.3 GFLOP)
     "c1_dense": dict(M=256, K=2048, N=4096, dense=True),
+    # BASELINE config 2: routing only (top-4 of 128 logits, softmax, histogram, gather / scatter indices, tables)
+    "c2_routing": dict(T=4096, E=128, k=4, routing=True),
+    # quantise / dequantise of weights in the matmul's layout: [8, 2880, 5760] float32 -> MXFP4 along K -> bfloat16
+    "quant": dict(E=8, K=2880, N=5760, quant=True),
+    "dequant": dict(E=8, K=2880, N=5760, dequant=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
     # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
     "hbm_copy": dict(bytes=1 << 30),
 }
+# the configurations BASELINE.json lists beside the headline one, and the pair that prepares / checks its weights
+CONFIG_RUNS = (("c1_dense", "c1_dense"), ("c2_routing", "c2_routing"), ("c4_decode", "fc1_decode"),
+               ("c5_fc2_combine", "fc2_combine"), ("quant", "quant"), ("dequant", "dequant"))
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# HBM traffic of the dominant kernels: measured with rocprofv3 counters outside this process and kept, with the digest
+# of the kernel sources it was measured on, in profiles/hbm_traffic.txt
+# ---------------------------------------------------------------------------------------------------------------------
+def kernel_sources_digest():
+    """sha256 over the kernel sources (csrc/*.h, *.hip, *.cpp and the C header), in name order."""
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "triton_amd", "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".h", ".hip", ".cpp")))
+    for path in files + [os.path.join(ROOT, "include", "triton_amd.h")]:
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """(bytes per launch or None, where the number comes from).  None when the committed profile holds no line for
+    the workload or was taken on other kernel sources than the ones in the tree."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, "profiles/hbm_traffic.txt is missing"
+    text = open(path).read()
+    m = re.search(r"kernel sources digest:\s*([0-9a-f]+)", text)
+    digest = kernel_sources_digest()
+    if not m or m.group(1) != digest:
+        return None, (f"profiles/hbm_traffic.txt was measured on kernel sources {m.group(1) if m else '?'}, the tree "
+                      f"holds {digest}: stale, not reported")
+    for line in text.splitlines():
+        lm = re.match(r"\S.*\((\w+)\)\s+([\d,]+)\s+([\d,]+)\s+([\d,]+)\s+([\d,]+)\s+([\d,]+)\s+([\d,]+)\s+[\d.]+\s*$", line)
+        if lm and lm.group(1) == workload and "mm_" in line:
+            return int(lm.group(6).replace(",", "")), ("profiles/hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                                       f"scaled by a copy kernel, kernel sources {digest})")
+    return None, "profiles/hbm_traffic.txt has no line for this workload"
+
+
+SPIN_UP_MS = 0.0  # set for the short runs of the other configurations (see main)
+
+
+def spin_up(fn):
+    """Keeps the GPU busy with `fn` for SPIN_UP_MS before a short timed run: after a pause on the host (an oracle
+    check of the previous configuration) the first milliseconds of GPU work run at idle clocks, which a run of a few
+    milliseconds would otherwise be measured in."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SPIN_UP_MS:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+
+
+def timed(fn, steps, warmup):
+    """Runs fn warmup + steps times; returns (results of the last call, mean HIP-event ms around a call, wall ms per call)."""
+    out = None
+    spin_up(fn)
+    for _ in range(warmup):
+        out = fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        a.record()
+        out = fn()
+        b.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return out, sum(a.elapsed_time(b) for a, b in ev) / steps, wall
+
+
+def base_line(args, metric, value, unit, ms_per_step, dtype, workload_text, **config):
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": dtype, "data": "synthetic", "config": {"workload": workload_text, **config}}
 
 
 def hbm_copy(args):
@@ -53,77 +135,14 @@ def hbm_copy(args):
     n = WORKLOADS["hbm_copy"]["bytes"] // 4
     src = torch.ones(n, dtype=torch.float32, device="cuda:0")
     dst = torch.empty_like(src)
-    for _ in range(args.warmup):
-        torch.mul(src, 1.0, out=dst)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for a, b in ev:
-        a.record()
-        torch.mul(src, 1.0, out=dst)
-        b.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    _, ms, wall = timed(lambda: torch.mul(src, 1.0, out=dst), args.steps, args.warmup)
     gbs = 2 * n * 4 / (ms * 1e-3) / 1e9
-    print(json.dumps({"metric": "hbm_copy_gbs", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-                      "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
-                      "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-                      "config": {"workload": f"hbm_copy: torch.mul(src, 1.0, out=dst), {n * 4} bytes read + written"},
-                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                   "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel_ms": round(ms, 4)},
-                      "cpu_baseline": None}))
-
-
-def run_dense(args, cfg):
-    """BASELINE config 1: y = x . deq(W) + bias, x bf16 [M, K], W MXFP4 [K, N] quantised along K."""
-    from oracle import matmul_ref as MR
-    from triton_amd.matmul import PrecisionConfig, matmul
-    M, K, N = cfg["M"], cfg["K"], cfg["N"]
-    dev = torch.device("cuda:0")
-    torch.manual_seed(0)
-    x_cpu = torch.randn(M, K).to(torch.bfloat16)
-    bias_cpu = (torch.randn(N) * 0.01).to(torch.bfloat16)
-    vals, scales = make_weights(1, K, N, dev)
-    vals, scales = vals[0], scales[0]
-    x, bias = x_cpu.to(dev), bias_cpu.to(dev)
-    pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
-    for _ in range(args.warmup):
-        y = matmul(x, vals, bias, precision_config=pc)
-    torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for a, b in events:
-        a.record()
-        y = matmul(x, vals, bias, precision_config=pc)
-        b.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
-    ms_per_step = wall * 1e3 / args.steps
-    flops = 2.0 * M * K * N
-    alg_bytes = M * K * 2 + K // 2 * N + K // 32 * N + N * 2 + M * N * 2
-    torch.set_num_threads(os.cpu_count())
-    t0 = time.perf_counter()
-    ref = MR.matmul_ref(x_cpu, vals.cpu(), bias_cpu, b_mx_scale=scales.cpu())
-    cpu_s = time.perf_counter() - t0
-    ok = bool(torch.allclose(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2))
-    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
-    print(json.dumps({
-        "metric": "moe_matmul_ogs_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x mxfp4 (fp32 accumulate)",
-        "data": "synthetic",
-        "config": {"workload": f"{args.workload}: dense matmul + bias, M={M}, K={K}, N={N}, W mxfp4 [{K},{N}]",
-                   "scale_layout": args.scale_layout},
-        "matmul_kernel_tflops": round(flops / (kernel_ms * 1e-3) / 1e12, 2),
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_stream16_kernel",
-                     "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes, "algorithmic_flops": flops,
-                     "note": "event pairs around one launch include launch latency; the problem is latency bound"},
-        "cpu_baseline": {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
-                         "sample": f"oracle matmul_ref on the whole problem, {cpu_s:.2f} s"},
-        "parity": {"gemm_within_1e-2": ok}}))
+    out = base_line(args, "hbm_copy_gbs", round(gbs, 1), "GB/s", wall, "f32",
+                    f"hbm_copy: torch.mul(src, 1.0, out=dst), {n * 4} bytes read + written")
+    out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel_ms": round(ms, 4)}
+    out["cpu_baseline"] = None
+    return out
 
 
 def make_weights(E, K, N, device, seed=0):
@@ -151,6 +170,127 @@ def scales_for_matmul(scales, layout):
     from triton_amd.tensor import convert_layout, wrap_torch_tensor
     from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
     return convert_layout(wrap_torch_tensor(scales), CDNA4MXScaleLayout())
+
+
+def run_dense(args, cfg, name):
+    """BASELINE config 1: y = x . deq(W) + bias, x bf16 [M, K], W fp32 [K, N] quantised to MXFP4 along K; the codes and
+    scales of that quantisation are checked against the oracle bit for bit on the way."""
+    from oracle import matmul_ref as MR
+    from oracle.mxfp_ref import downcast_to_mxfp_ref
+    from triton_amd.matmul import PrecisionConfig, matmul
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+    M, K, N = cfg["M"], cfg["K"], cfg["N"]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    x_cpu = torch.randn(M, K).to(torch.bfloat16)
+    bias_cpu = (torch.randn(N) * 0.01).to(torch.bfloat16)
+    w_cpu = torch.randn(K, N) * 0.02
+    vals, scales = downcast_to_mxfp(w_cpu.to(dev), torch.uint8, axis=0)
+    rv, rs = downcast_to_mxfp_ref(w_cpu, torch.uint8, 0)
+    codes_ok = bool(torch.equal(vals.cpu(), rv) and torch.equal(scales.cpu(), rs))
+    x, bias = x_cpu.to(dev), bias_cpu.to(dev)
+    pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
+    y, kernel_ms, wall = timed(lambda: matmul(x, vals, bias, precision_config=pc), args.steps, args.warmup)
+    flops = 2.0 * M * K * N
+    alg_bytes = M * K * 2 + K // 2 * N + K // 32 * N + N * 2 + M * N * 2
+    torch.set_num_threads(os.cpu_count())
+    t0 = time.perf_counter()
+    ref = MR.matmul_ref(x_cpu, vals.cpu(), bias_cpu, b_mx_scale=scales.cpu())
+    cpu_s = time.perf_counter() - t0
+    ok = bool(torch.allclose(y.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2))
+    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    out = base_line(args, "moe_matmul_ogs_tflops", round(flops / (wall * 1e-3) / 1e12, 2), "TFLOP/s", wall,
+                    "bf16 x mxfp4 (fp32 accumulate)",
+                    f"{name}: dense matmul + bias, M={M}, K={K}, N={N}, W mxfp4 [{K},{N}]", scale_layout=args.scale_layout)
+    out["matmul_kernel_tflops"] = round(flops / (kernel_ms * 1e-3) / 1e12, 2)
+    out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_stream16_kernel",
+                       "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes, "algorithmic_flops": flops,
+                       "note": "event pairs around one call include its host time; the problem is latency bound "
+                               "(4.3 GFLOP, 7.6 MB)"}
+    out["cpu_baseline"] = {"value": round(flops / cpu_s / 1e12, 4), "unit": "TFLOP/s", "cores": os.cpu_count(),
+                           "kind": "port", "sample": f"oracle matmul_ref on the whole problem, {cpu_s:.2f} s"}
+    out["parity"] = {"gemm_within_1e-2": ok, "mxfp4_codes_and_scales_bit_exact": codes_ok}
+    return out
+
+
+def run_routing(args, cfg, name):
+    """BASELINE config 2: routing(logits) alone.  Bit-exact integers against the oracle; launch-latency bound."""
+    from oracle import routing_ref as RR
+    from triton_amd.routing import routing
+    T, E, k = cfg["T"], cfg["E"], cfg["k"]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    logits_cpu = torch.randn(T, E)
+    logits = logits_cpu.to(dev)
+    r, kernel_ms, wall = timed(lambda: routing(logits, k), args.steps, args.warmup)
+    t0 = time.perf_counter()
+    ref = RR.routing_ref(logits_cpu, k)
+    cpu_s = time.perf_counter() - t0
+    rm, rr = r.ragged_metadata, ref["ragged"]
+    ok = bool(torch.equal(r.indx.cpu().int(), ref["indx"]) and torch.equal(r.col_sum.cpu(), ref["col_sum"])
+              and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]) and torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"])
+              and torch.equal(r.row_sorted_indx.cpu(), ref["row_sorted_indx"]) and torch.equal(rm.slice_offs.cpu(), rr.slice_offs)
+              and torch.equal(rm.block_offs_data.cpu(), rr.block_offs_data)
+              and torch.equal(rm.block_schedule_data.cpu(), rr.block_schedule_data))
+    vals_ok = bool(torch.allclose(r.vals.cpu(), ref["vals"], rtol=1e-5, atol=1e-7))
+    # logits in; indices, values, bit matrix, histogram, three index arrays and the tables out
+    alg_bytes = T * E * 4 + T * k * (2 + 4) + T * ((E + 31) // 32) * 4 + E * 4 + 3 * T * k * 4 + 6 * (E + 1) * 4
+    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    out = base_line(args, "moe_routing_tokens_per_s", round(T / (wall * 1e-3), 1), "tokens/s", wall, "f32 logits -> int32",
+                    f"{name}: routing (top-{k} of {E} + softmax, histogram, gather / scatter indices, ragged tables), T={T}")
+    out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "topk_kernel + 3 metadata kernels",
+                       "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes,
+                       "note": "2.4 MB in four launches: bound by launch latency, not by HBM"}
+    out["cpu_baseline"] = {"value": round(T / cpu_s, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
+                           "sample": f"oracle routing_ref (numpy) on the whole batch, {cpu_s:.3f} s"}
+    out["parity"] = {"routing_bit_exact": ok, "softmax_values_within_1e-5": vals_ok}
+    return out
+
+
+def run_quant(args, cfg, name):
+    """Weights [E, K, N] float32 -> MXFP4 along K (the layout the matmul consumes), and back to bfloat16.  HBM bound:
+    achieved = (source bytes + codes + scales) / kernel time."""
+    from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp, upcast_from_mxfp
+    E, K, N = cfg["E"], cfg["K"], cfg["N"]
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    w = torch.randn((E, K, N), generator=g, device=dev, dtype=torch.float32) * 0.02
+    n = E * K * N
+    sample = w[:1, :, :256].cpu()  # the oracle checks one expert's first 256 columns (bit-exact)
+    if cfg.get("quant"):
+        (v, s), kernel_ms, wall = timed(lambda: downcast_to_mxfp(w, torch.uint8, axis=1), args.steps, args.warmup)
+        alg_bytes = n * 4 + n // 2 + n // 32
+        t0 = time.perf_counter()
+        rv, rs = downcast_to_mxfp_ref(sample, torch.uint8, 1)
+        cpu_s = time.perf_counter() - t0
+        ok = bool(torch.equal(v[:1, :, :256].cpu(), rv) and torch.equal(s[:1, :, :256].cpu(), rs))
+        what, kern, dtype = "downcast_to_mxfp: float32 -> e2m1 codes + e8m0 scales", "downcast_cols_kernel", "f32 -> mxfp4"
+        parity = {"codes_and_scales_bit_exact": ok}
+    else:
+        v, s = downcast_to_mxfp(w, torch.uint8, axis=1)
+        y, kernel_ms, wall = timed(lambda: upcast_from_mxfp(v, s, torch.bfloat16, axis=1), args.steps, args.warmup)
+        alg_bytes = n // 2 + n // 32 + n * 2
+        vs, ss = v[:1, :, :256].cpu(), s[:1, :, :256].cpu()
+        t0 = time.perf_counter()
+        ref = upcast_from_mxfp_ref(vs, ss, torch.bfloat16, 1)
+        cpu_s = time.perf_counter() - t0
+        ok = bool(torch.equal(y[:1, :, :256].cpu().view(torch.int16), ref.view(torch.int16)))
+        what, kern, dtype = "upcast_from_mxfp: e2m1 codes + e8m0 scales -> bfloat16", "upcast_cols_kernel", "mxfp4 -> bf16"
+        parity = {"values_bit_exact": ok}
+    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    out = base_line(args, "mxfp_gbs", round(alg_bytes / (wall * 1e-3) / 1e9, 1), "GB/s", wall, dtype,
+                    f"{name}: {what}, weights [{E},{K},{N}] quantised along K")
+    out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": kern,
+                       "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes}
+    out["cpu_baseline"] = {"value": round(sample.numel() * (alg_bytes / n) / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1,
+                           "kind": "port", "sample": f"oracle (numpy) on one expert's first 256 columns, {cpu_s:.2f} s"}
+    out["parity"] = parity
+    return out
 
 
 def algorithmic_bytes(col_sum, T, k, K, N, act):
@@ -186,8 +326,16 @@ def cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, experts, K, N, act, fc2=Non
     return y, n_rows, flops / dt / 1e12, dt
 
 
-def run_fc2(args, cfg):
+def sample_experts(args, rows, E, K, N):
+    """Experts in the CPU sample: as asked, or about 0.6 TFLOP of oracle work (10-15 s on the box's host cores)."""
+    if args.cpu_experts > 0:
+        return min(args.cpu_experts, E)
+    return max(1, min(E, int(6e11 * args.cpu_work / (2.0 * rows / E * K * N))))
+
+
+def run_fc2(args, cfg, name):
     """BASELINE config 5: y = scatter((x8 . deq(W2[e]) * sx + bias[e]) * gate), z = sum over the k slots."""
+    from oracle import matmul_ref as MR
     from oracle import routing_ref as RR
     from triton_amd.matmul import FlexCtx, InFlexData, PrecisionConfig, matmul
     from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
@@ -221,14 +369,18 @@ def run_fc2(args, cfg):
         y = matmul(x8, vals, bias, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam, c=y_buf)
         if ev is not None:
             ev[1].record()
+            ev[2].record()
         z, _ = reduce(y.view(T, k, N), dim=1)
+        if ev is not None:
+            ev[3].record()
         return r, gam, y, z
 
     with scoped_opt_flags_constraints(constraints):
+        spin_up(step)
         for _ in range(args.warmup):
             r, gam, y, z = step()
         torch.cuda.synchronize()
-        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(args.steps):
@@ -236,36 +388,41 @@ def run_fc2(args, cfg):
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    kernel_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    combine_ms = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
     flops = 2.0 * rows * K * N
     col_sum = r.col_sum.cpu()
     n_active = int((col_sum > 0).sum())
     mm_bytes = rows * K + n_active * (K // 2 * N + K // 32 * N + N * 2) + rows * 8 + rows * N * 2
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
     gbs_kernel = mm_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic, traffic_source = measured_traffic(name)
     if rows <= 16 * E:  # decode size: weight streaming, bound by HBM
         roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
+                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=traffic, traffic_source=traffic_source,
                     kernel="mm_stream16_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
                     algorithmic_flops=flops)
     else:
         roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=PEAK_FP8_TFLOPS, unit="TFLOP/s",
-                    frac=round(tflops_kernel / PEAK_FP8_TFLOPS, 4), traffic=MEASURED_TRAFFIC.get(args.workload),
+                    frac=round(tflops_kernel / PEAK_FP8_TFLOPS, 4), traffic=traffic, traffic_source=traffic_source,
                     kernel="mm_x8_mxfp4_kernel", kernel_ms=round(kernel_ms, 4), algorithmic_bytes=mm_bytes,
                     algorithmic_flops=flops, frac_of_mxfp4_peak=round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4),
                     hbm_gbs=round(gbs_kernel, 1))
+    combine_bytes = rows * N * 2 + T * N * 2
+    roof["combine"] = dict(kernel="reduce_kernel", kernel_ms=round(combine_ms, 4), bound="hbm", algorithmic_bytes=combine_bytes,
+                           achieved=round(combine_bytes / (combine_ms * 1e-3) / 1e9, 1), unit="GB/s",
+                           frac=round(combine_bytes / (combine_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4))
     ref = RR.routing_ref(logits_cpu, k)
     routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(col_sum, ref["col_sum"]))
     gam_ref = ref["vals"].flatten()[ref["col_sorted_indx"].long()]
     routing_ok = routing_ok and bool(torch.allclose(gam.cpu(), gam_ref, rtol=1e-5, atol=1e-7))  # softmax values
     gam_ref = gam.cpu()
     # the combine is a fixed-order fp32 sum: bit-exact given y
-    from oracle import matmul_ref as MR
-    n_chk = 2048
+    n_chk = min(2048, T)
     combine_ok = bool(torch.equal(z[:n_chk].cpu(), MR.reduce_ref(y.view(T, k, N)[:n_chk].cpu(), 1)))
     cpu, gemm_ok = None, None
     if args.cpu_experts != 0:
-        n_e = min(args.cpu_experts, E) if args.cpu_experts > 0 else max(1, min(E, int(6e11 / (2.0 * rows / E * K * N))))
+        n_e = sample_experts(args, rows, E, K, N)
         y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x8.cpu(), vals, scales, bias_cpu, ref, n_e, K, N, False,
                                                         fc2=(x_scale.cpu(), gam_ref))
         got = y.cpu()[ref["scatter_indx"][:n_rows].long()]
@@ -273,60 +430,26 @@ def run_fc2(args, cfg):
         cpu = dict(value=round(cpu_tflops, 5), unit="TFLOP/s", cores=os.cpu_count(), kind="port",
                    sample=f"oracle matmul_ref (dequantise + fp32 GEMM, gate weights) on the first {n_e} of {E} experts "
                           f"({n_rows} of {rows} rows), {cpu_s:.1f} s")
-    print(json.dumps({
-        "metric": "moe_matmul_ogs_tflops", "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8e4m3 x mxfp4 (fp32 accumulate)",
-        "data": "synthetic",
-        "config": {"workload": f"{args.workload}: routing + matmul_ogs(fp8 rows, grouped GEMM, bias, gate weights, scatter) + "
-                               f"top-{k} combine, T={T}, hidden={K}, experts={E}, W2 mxfp4 [{E},{K},{N}]",
-                   "rows": rows, "active_experts": n_active, "scale_layout": args.scale_layout},
-        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
-        "roofline": roof, "cpu_baseline": cpu,
-        "parity": {"routing_bit_exact": routing_ok, "combine_bit_exact": combine_ok, "gemm_sample_within_1e-2": gemm_ok},
-    }))
+    out = base_line(args, "moe_matmul_ogs_tflops", round(flops / (ms_per_step * 1e-3) / 1e12, 2), "TFLOP/s", ms_per_step,
+                    "fp8e4m3 x mxfp4 (fp32 accumulate)",
+                    f"{name}: routing + matmul_ogs(fp8 rows, grouped GEMM, bias, gate weights, scatter) + "
+                    f"top-{k} combine, T={T}, hidden={K}, experts={E}, W2 mxfp4 [{E},{K},{N}]",
+                    rows=rows, active_experts=n_active, scale_layout=args.scale_layout)
+    out.update({"tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
+                "roofline": roof, "cpu_baseline": cpu,
+                "parity": {"routing_bit_exact": routing_ok, "combine_bit_exact": combine_ok,
+                           "gemm_sample_within_1e-2": gemm_ok}})
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="fc1_prefill", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-experts", type=int, default=-1,
-                    help="experts in the CPU baseline sample (0 = skip; default: about 0.6 TFLOP of oracle work, 10-15 s)")
-    ap.add_argument("--block-m", type=int, default=0)
-    ap.add_argument("--scale-layout", default="strided", choices=["strided", "cdna4"],
-                    help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
-                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout()))")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (with more GPUs the experts "
-              "would be sharded across them, one exchange of rows before and after the two matmuls)", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
-        sys.exit(3)
-
-    if args.workload == "hbm_copy":
-        hbm_copy(args)
-        return
-
-    if WORKLOADS[args.workload].get("dense"):
-        run_dense(args, WORKLOADS[args.workload])
-        return
-
-    if WORKLOADS[args.workload].get("fc2"):
-        run_fc2(args, WORKLOADS[args.workload])
-        return
-
+def run_fc1(args, cfg, name):
+    """BASELINE configs 3 / 4: routing + matmul_ogs(gather, grouped GEMM, bias + SwiGLU)."""
     from oracle import routing_ref as RR
     from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
     from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
     from triton_amd.routing import routing
     from triton_amd.swiglu import swiglu_fn
 
-    cfg = WORKLOADS[args.workload]
     T, E, k, K, N, act = cfg["T"], cfg["E"], cfg["k"], cfg["K"], cfg["N"], cfg["act"]
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
@@ -359,17 +482,15 @@ def main():
         return r, y
 
     with scoped_opt_flags_constraints(constraints):
+        spin_up(step)
         for _ in range(args.warmup):
             r, y = step()
         torch.cuda.synchronize()
         events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        start.record()
         for i in range(args.steps):
             r, y = step(events[i])
-        stop.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -384,12 +505,13 @@ def main():
     gbs_kernel = abytes / (kernel_ms * 1e-3) / 1e9
     peak_mfma = PEAK_FP8_TFLOPS if mx8 else PEAK_BF16_TFLOPS
     hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (peak_mfma * 1e12))
+    traffic, traffic_source = measured_traffic(name)
     if hbm_bound:
         roof = dict(bound="hbm", achieved=round(gbs_kernel, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
+                    frac=round(gbs_kernel / PEAK_HBM_GBS, 4), traffic=traffic, traffic_source=traffic_source)
     else:
         roof = dict(bound="mfma", achieved=round(tflops_kernel, 1), peak=peak_mfma, unit="TFLOP/s",
-                    frac=round(tflops_kernel / peak_mfma, 4), traffic=MEASURED_TRAFFIC.get(args.workload))
+                    frac=round(tflops_kernel / peak_mfma, 4), traffic=traffic, traffic_source=traffic_source)
     # row blocks of 16 (few rows per expert) run the weight-streaming kernel, everything else the tiled one
     roof["kernel"] = "mm_stream16_kernel" if rows <= 16 * E else ("mm_x8_mxfp4_kernel" if mx8 else "mm_x16_mxfp4_kernel")
     roof["kernel_ms"] = round(kernel_ms, 4)
@@ -411,7 +533,7 @@ def main():
     cpu = None
     gemm_ok = None
     if args.cpu_experts != 0:
-        n_e = min(args.cpu_experts, E) if args.cpu_experts > 0 else max(1, min(E, int(6e11 / (2.0 * rows / E * K * N))))
+        n_e = sample_experts(args, rows, E, K, N)
         x_ref = x_cpu
         if mx8:  # the oracle sees the same quantised activations, dequantised (exactly) to bf16
             from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
@@ -422,21 +544,84 @@ def main():
         cpu = dict(value=round(cpu_tflops, 5), unit="TFLOP/s", cores=os.cpu_count(), kind="port",
                    sample=f"oracle matmul_ref (dequantise + fp32 GEMM + SwiGLU) on the first {n_e} of {E} experts "
                           f"({n_rows} of {rows} rows), {cpu_s:.1f} s")
-    out = {
-        "metric": "moe_matmul_ogs_tflops", "value": round(tflops_step, 2), "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None,
-        "dtype": ("mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") + " (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: routing + " + ("downcast_to_mxfp(x) + " if mx8 else "") +
-                               f"matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, "
-                               f"hidden={K}, experts={E}, top-{k}, W1 mxfp4 [{E},{K},{N}]",
-                   "rows": rows, "active_experts": n_active, "scale_layout": args.scale_layout},
-        "tokens_per_s": round(T / (ms_per_step * 1e-3), 1),
-        "matmul_kernel_tflops": round(tflops_kernel, 2),
-        "roofline": roof,
-        "cpu_baseline": cpu,
-        "parity": {"routing_bit_exact": routing_ok, "gemm_sample_within_1e-2": gemm_ok},
-    }
+    out = base_line(args, "moe_matmul_ogs_tflops", round(tflops_step, 2), "TFLOP/s", ms_per_step,
+                    ("mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") + " (fp32 accumulate)",
+                    f"{name}: routing + " + ("downcast_to_mxfp(x) + " if mx8 else "") +
+                    f"matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, hidden={K}, experts={E}, top-{k}, "
+                    f"W1 mxfp4 [{E},{K},{N}]", rows=rows, active_experts=n_active, scale_layout=args.scale_layout)
+    out.update({"tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
+                "roofline": roof, "cpu_baseline": cpu,
+                "parity": {"routing_bit_exact": routing_ok, "gemm_sample_within_1e-2": gemm_ok}})
+    return out
+
+
+def run_workload(args, name):
+    cfg = WORKLOADS[name]
+    if name == "hbm_copy":
+        return hbm_copy(args)
+    if cfg.get("dense"):
+        return run_dense(args, cfg, name)
+    if cfg.get("routing"):
+        return run_routing(args, cfg, name)
+    if cfg.get("quant") or cfg.get("dequant"):
+        return run_quant(args, cfg, name)
+    if cfg.get("fc2"):
+        return run_fc2(args, cfg, name)
+    return run_fc1(args, cfg, name)
+
+
+def config_summary(line):
+    """What the headline line carries of another configuration's run."""
+    r = line["roofline"]
+    s = {"workload": line["config"]["workload"], "ms_per_step": line["ms_per_step"], "kernel": r.get("kernel"),
+         "kernel_ms": r["kernel_ms"], "bound": r["bound"], "achieved": r["achieved"], "unit": r["unit"], "peak": r["peak"],
+         "frac": r["frac"], "parity": line.get("parity")}
+    for key in ("combine", "note", "traffic"):
+        if r.get(key) is not None:
+            s[key] = r[key]
+    if line.get("tokens_per_s") is not None:
+        s["tokens_per_s"] = line["tokens_per_s"]
+    return s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="fc1_prefill", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-experts", type=int, default=-1,
+                    help="experts in the CPU baseline sample (0 = skip; default: about 0.6 TFLOP of oracle work, 10-15 s)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload only: leave out the short runs of the other configurations")
+    ap.add_argument("--block-m", type=int, default=0)
+    ap.add_argument("--scale-layout", default="strided", choices=["strided", "cdna4"],
+                    help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
+                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout()))")
+    args = ap.parse_args()
+    args.cpu_work = 1.0
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (with more GPUs the experts "
+              "would be sharded across them, one exchange of rows before and after the two matmuls)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+
+    out = run_workload(args, args.workload)
+    if args.workload == "fc1_prefill" and not args.no_configs:
+        # the other configurations: fewer steps, and a tenth of the oracle work in their parity samples
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup, sub.cpu_work = min(args.steps, 10), min(args.warmup, 3), 0.1
+        global SPIN_UP_MS
+        SPIN_UP_MS = 100.0
+        configs = {}
+        for key, name in CONFIG_RUNS:
+            t0 = time.perf_counter()
+            configs[key] = config_summary(run_workload(sub, name))
+            configs[key]["bench_seconds"] = round(time.perf_counter() - t0, 1)
+            torch.cuda.empty_cache()
+        out["configs"] = configs
     print(json.dumps(out))
 
 
