@@ -265,6 +265,53 @@ int tamd_reduce(const void *x, int x_dtype, int64_t S0, int64_t R, int64_t S1, i
                 int64_t ys0, int64_t ys1, void *stream);
 
 /*
+ * General reduction over the middle axis: replaces the launch of _reduce_forward with all of its optional operands
+ * (reduce.py:375-492 kernel body, :818-957 host, API :1135-1157).  x [S0, R, S1] -> y [S0, S1 / n] where n = 1
+ * without post-processing and 2 with one of the pairwise functions below.
+ *
+ *   acc[s0, c] = sum_r mask * (x * 2^(x_mx_scale - 127) * *x_flex_scale * scale)       float32, r in index order
+ *   o          = postprocess(acc) * *x_global_scale
+ *   flexpoint output (no y_mx_scale): *y_actual_scale <- max(*y_actual_scale, max|o| / max_finite(y_dtype) + 1e-30)
+ *                                     by atomic max; o / *y_expected_scale, clamped to y_dtype's finite range when
+ *                                     y_saturate_inf; cast (numerics_details/flexpoint.py:137-188)
+ *   MXFP8 output (y_mx_scale given):  o / *y_expected_scale quantised per 32 output columns exactly as
+ *                                     tamd_downcast_mxfp (ROUND_UP, float8_e4m3fn values) quantises float32 input
+ * x_dtype / y_dtype: F32, F16, BF16, FP8_E4M3, FP8_E5M2.  x_mx_scale: e8m0 bytes, one per 32 columns of S1, indexed
+ * [s0, r, c / 32] with its own strides.  mask (nonzero = keep) and scale (float32) are indexed with their own
+ * strides (0 broadcasts).  Every pointer but x and y may be NULL.
+ */
+#define TAMD_PP_NONE 0
+#define TAMD_PP_SWIGLU 1          /* o[j] = swiglu(acc[2j], acc[2j+1]; alpha = pp_arg0, limit = pp_arg1 if pp_has_arg1) */
+#define TAMD_PP_PLUS_A_PAIRSUM 2  /* o[j] = (acc[2j] + pp_arg0) + (acc[2j+1] + pp_arg0): tests/test_reduce.py:35-38 */
+typedef struct tamd_reduce_args {
+  const void *x;
+  int x_dtype;
+  int64_t S0, R, S1;
+  int64_t xs0, xsr, xs1;
+  const uint8_t *x_mx_scale;
+  int64_t xms0, xmsr, xms1;
+  const float *x_flex_scale;
+  const float *x_global_scale;
+  const uint8_t *mask;
+  int64_t ms0, msr, ms1;
+  const float *scale;
+  int64_t ss0, ssr, ss1;
+  int postprocess; /* TAMD_PP_* */
+  float pp_arg0, pp_arg1;
+  int pp_has_arg1;
+  void *y;
+  int y_dtype;
+  int64_t ys0, ys1;
+  const float *y_expected_scale;
+  float *y_actual_scale;
+  int y_saturate_inf;
+  uint8_t *y_mx_scale; /* [S0, ceil(S1 / n / 32)] */
+  int64_t yms0, yms1;
+} tamd_reduce_args;
+
+int tamd_reduce_ex(const tamd_reduce_args *args, void *stream);
+
+/*
  * standalone interleaved SwiGLU: replaces the launch of _swiglu (swiglu.py:52-76).
  * a [M, 2*N_out] -> out [M, N_out].
  */

@@ -133,3 +133,55 @@ def reduce_mx_ref(x: torch.Tensor, x_mxscale: torch.Tensor, dim: int, mask=None,
     for r in range(xf.shape[dim]):
         acc = acc + xf.select(dim, r)
     return downcast_to_mxfp_ref(acc, torch.float8_e4m3fn, axis=-1)
+
+
+_MAX_FINITE = {torch.float8_e4m3fn: 448.0, torch.float8_e5m2: 57344.0, torch.float16: 65504.0,
+               torch.bfloat16: 3.3895313892515355e38, torch.float32: 3.4028234663852886e38}
+
+
+def reduce_general_ref(x: torch.Tensor, dim: int, mask=None, scale=None, x_mxscale=None, x_flex_scale=None,
+                       x_global_scale=None, postprocess=None, y_dtype=None, y_expected_scale=None,
+                       y_saturate_inf: bool = False, y_has_mx: bool = False):
+    """reduce_torch (reduce.py:1179-1210 of the reference) together with the operands only its kernel has
+    (_reduce_forward_inner, reduce.py:441-492): the order of the factors of a term ((x * 2^e) * x_flex_scale) * scale,
+    x_global_scale after the post-processing function, the flexpoint output as float_to_flex computes it
+    (numerics_details/flexpoint.py:137-188: actual scale = max|y| / max_finite + 1e-30, y * (1 / expected), clamp when
+    saturating).  Built from pieces that are pinned on their own -- upcast_from_mxfp_ref, swiglu_ref,
+    downcast_to_mxfp_ref, torch's casts -- around an explicit index-order float32 sum.
+
+    postprocess: None, ("swiglu", alpha, limit) or ("plus_a", a).  Returns (y, y_mxscale or None, actual_scale)."""
+    from .mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+    y_dtype = y_dtype or x.dtype
+    xf = upcast_from_mxfp_ref(x, x_mxscale, torch.float32, axis=-1) if x_mxscale is not None else x.to(torch.float32)
+    if x_flex_scale is not None:
+        xf = xf * x_flex_scale.to(torch.float32)
+    if scale is not None:
+        xf = xf * scale.to(torch.float32)
+    if mask is not None:
+        xf = torch.where(mask.to(torch.bool), xf, torch.zeros((), dtype=torch.float32))
+    dim = dim % xf.ndim
+    acc = torch.zeros([n for i, n in enumerate(xf.shape) if i != dim], dtype=torch.float32)
+    for r in range(xf.shape[dim]):
+        acc = acc + xf.select(dim, r)
+    if postprocess is not None:
+        if postprocess[0] == "swiglu":
+            acc = swiglu_ref(acc, postprocess[1], postprocess[2])
+        elif postprocess[0] == "plus_a":
+            t = acc + torch.tensor(postprocess[1], dtype=torch.float32)
+            acc = t[..., 0::2] + t[..., 1::2]
+        else:
+            raise ValueError(postprocess[0])
+    if x_global_scale is not None:
+        acc = acc * x_global_scale.to(torch.float32)
+    max_finite = _MAX_FINITE[torch.float8_e4m3fn if y_has_mx else y_dtype]
+    absmax = acc.abs().max() if acc.numel() else torch.zeros(())
+    absmax = torch.where(torch.isnan(absmax), torch.tensor(float("inf")), absmax)
+    actual = (absmax * torch.tensor(1.0 / max_finite, dtype=torch.float32) + torch.tensor(1.0e-30, dtype=torch.float32)).reshape(1)
+    if y_expected_scale is not None:
+        acc = acc * (torch.ones((), dtype=torch.float32) / y_expected_scale.to(torch.float32))
+        if y_saturate_inf and not y_has_mx:
+            acc = acc.clamp(-max_finite, max_finite)
+    if y_has_mx:
+        v, s = downcast_to_mxfp_ref(acc, torch.float8_e4m3fn, axis=-1)
+        return v, s, actual
+    return acc.to(y_dtype), None, actual

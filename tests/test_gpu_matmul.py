@@ -799,6 +799,38 @@ def test_split_k_refuses_what_it_cannot_do(device):
             matmul(x, v, None, md, scatter_indx=scatter, precision_config=pc)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float8_e4m3fn, torch.bfloat16])
+@pytest.mark.parametrize("act", [False, True])
+def test_split_k_with_flexpoint_output(out_dtype, act, device):
+    """The ranges' float32 partial sums are finished by ONE reduction launch that applies the fused activation and the
+    output's flexpoint scales (matmul.py:711-737 of the reference): same numbers as the unsplit kernel's epilogue."""
+    from triton_amd.matmul import FlexCtx, OutFlexData
+    torch.manual_seed(5)
+    M, K, N = 48, 1024, 256
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = torch.randn(K, N) * 0.02
+    bias = torch.randn(N)
+    v, s, rv, rs = quantize_w(w, device)
+    fa = swiglu_act(1.702, 7.0) if act else None
+    expected = torch.tensor([0.05])
+    outs = []
+    for split in (1, 4):
+        actual = torch.zeros(1, device=device)
+        pc = PrecisionConfig(b_mx_scale=s, b_microblock_size=32, out_dtype=out_dtype, flexpoint_saturate_inf=True,
+                             flex_ctx=FlexCtx(out_data=OutFlexData(expected_scale=expected.to(device), actual_scale=actual)))
+        with scoped_opt_flags_constraints({"split_k": split} if split > 1 else {}):
+            y = matmul(x.to(device), v, bias.to(device), precision_config=pc, fused_activation=fa)
+        outs.append((y.cpu().float(), actual.cpu()))
+    (y1, a1), (y4, a4) = outs
+    torch.testing.assert_close(a4, a1, rtol=1e-3, atol=0)
+    # fp8 outputs: one step of the type (1/8 relative) where the two summation orders round apart
+    tol = dict(rtol=0.13, atol=0.5) if out_dtype == torch.float8_e4m3fn else dict(rtol=2e-2, atol=2e-1)
+    torch.testing.assert_close(y4, y1, **tol)
+    ref = MR.matmul_ref(x, rv, bias, b_mx_scale=rs, fused_swiglu=(1.702, 7.0) if act else None).float() / 0.05
+    ref = ref.clamp(-448.0, 448.0) if out_dtype == torch.float8_e4m3fn else ref
+    torch.testing.assert_close(y4, ref.to(out_dtype).float(), **tol)
+
+
 @pytest.mark.parametrize("kind", ["mxfp4", "bf16"])
 def test_long_k_with_few_rows_splits_by_itself(kind, device):
     """No constraint given: a dense problem with few rows and K >= 8192 is split without being asked."""

@@ -71,8 +71,7 @@ def test_reduce_mxfp8_in_and_out(shape, dim, mask_mode, use_scale, use_flex, dev
     yv, ys = reduce(xv.to(device), dim, mask=None if mask is None else mask.to(device),
                     scale=None if scale is None else scale.to(device), x_mxscale=xs.to(device),
                     x_flex=InFlexData(dtype=torch.float8_e4m3fn, scale=fscale.to(device)) if use_flex else InFlexData())
-    rv, rs = MR.reduce_mx_ref(xv, xs, dim, mask=mask, scale=None if scale is None else (scale * 0.75 if use_flex else scale),
-                              x_flex_scale=None)
+    rv, rs = MR.reduce_mx_ref(xv, xs, dim, mask=mask, scale=scale, x_flex_scale=fscale)
     assert yv.dtype == torch.float8_e4m3fn and torch.equal(ys.cpu(), rs)
     assert torch.equal(yv.cpu().view(torch.uint8), rv.contiguous().view(torch.uint8))
 
@@ -89,3 +88,116 @@ def test_reduce_long_axis(shape, dim, dtype, device):
     assert y.dtype == dtype and tuple(y.shape) == tuple(ref.shape)
     tol = dict(rtol=1e-2, atol=5e-1) if dtype != torch.float32 else dict(rtol=1e-4, atol=1e-3)
     torch.testing.assert_close(y.cpu().float(), ref.float(), **tol)
+
+
+# ---------------------------------------------------------------------------- the general reduction
+# after tests/test_reduce.py:41-120 of the reference (shapes scaled to what the CPU oracle sums in a second)
+
+def _init_mask(mode, B, M, N):
+    if mode == "none":
+        return None
+    shape = {"full": (B, M, N), "broadcast_b": (1, M, N), "broadcast_m": (B, 1, N), "broadcast_n": (B, M, 1)}[mode]
+    return torch.rand(shape) > 0.3
+
+
+@pytest.mark.parametrize("B,M,N,postprocess", [(31, 384, 96, None), (64, 31, 384, None), (48, 64, 311, None), (64, 64, 128, None),
+                                               (64, 64, 128, "plus_ten"), (64, 64, 128, "swiglu"), (4, 4, 4, None), (3, 15, 25, None),
+                                               (5, 999, 235, None), (15, 345, 78, "plus_ten")])
+@pytest.mark.parametrize("dtype_str", ["float16", "bfloat16", "float32", "mxfloat8", "flexfloat8_e4m3fn", "flexfloat8_e5m2"])
+@pytest.mark.parametrize("mask_mode", ["none", "full", "broadcast_b", "broadcast_m", "broadcast_n"])
+@pytest.mark.parametrize("dim", [0, 1, 2])
+def test_reduce_general(B, M, N, postprocess, dtype_str, mask_mode, dim, device):
+    from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
+    from triton_amd.numerics import InFlexData, OutFlexData
+    from triton_amd.reduce import PostprocessFn, plus_a_reduce
+    from triton_amd.specialize import FnSpecs
+    from triton_amd.swiglu import swiglu_fn
+    if mask_mode not in ("none", "full") and (B, M, N) not in ((64, 64, 128), (3, 15, 25), (48, 64, 311)):
+        pytest.skip("broadcast masks are exercised on three of the shapes")
+    torch.manual_seed(0)
+    x = torch.randn(B, M, N)
+    is_mx, is_flex = dtype_str.startswith("mx"), dtype_str.startswith("flex")
+    xs = fscale = expected = None
+    if is_mx:
+        x, xs = downcast_to_mxfp_ref(x.to(torch.float16), torch.float8_e4m3fn, axis=-1)
+        x, xs = x.contiguous(), xs.contiguous()
+    elif is_flex:
+        dt = getattr(torch, dtype_str.removeprefix("flex"))
+        fscale, expected = torch.tensor([2.0]), torch.tensor([4.0])
+        x = (x / fscale).to(dt)
+    else:
+        x = x.to(getattr(torch, dtype_str))
+    mask = _init_mask(mask_mode, B, M, N)
+    if dim == 2 and is_mx:
+        with pytest.raises(ValueError):
+            reduce(x.to(device), dim=dim, mask=None if mask is None else mask.to(device), x_mxscale=xs.to(device))
+        return
+    pp_tri, pp_ref = None, None
+    if postprocess is not None:
+        if dim == 2 or [B, M, N][2] % 2:
+            pytest.skip("the post-processing functions pair up columns of the last axis")
+        if postprocess == "plus_ten":
+            pp_tri, pp_ref = PostprocessFn(FnSpecs("plus_a", plus_a_reduce, ("a", ), reduction_n=2), (10, )), ("plus_a", 10.0)
+        else:
+            pp_tri = PostprocessFn(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0))
+            pp_ref = ("swiglu", 1.702, 7.0)
+    actual = torch.zeros(1, device=device)
+    y, y_mx = reduce(x.to(device), dim=dim, mask=None if mask is None else mask.to(device),
+                     x_mxscale=None if xs is None else xs.to(device),
+                     x_flex=InFlexData(scale=fscale.to(device)) if is_flex else InFlexData(),
+                     y_flex=OutFlexData(expected_scale=expected.to(device), actual_scale=actual) if is_flex else OutFlexData(),
+                     postprocess_fn1=pp_tri)
+    ry, ry_mx, ractual = MR.reduce_general_ref(x, dim, mask=mask, x_mxscale=xs, x_flex_scale=fscale, postprocess=pp_ref,
+                                               y_expected_scale=expected, y_has_mx=is_mx)
+    assert y.dtype == x.dtype and tuple(y.shape) == tuple(ry.shape)
+    if is_mx:
+        # bit-exact unless the post-processing function's transcendental differs in the last place
+        if postprocess == "swiglu":
+            a = upcast_from_mxfp_ref(y.cpu(), y_mx.cpu(), torch.float32, axis=-1)
+            b = upcast_from_mxfp_ref(ry, ry_mx, torch.float32, axis=-1)
+            torch.testing.assert_close(a, b, rtol=0.13, atol=1e-3)
+        else:
+            assert torch.equal(y_mx.cpu(), ry_mx)
+            assert torch.equal(y.cpu().view(torch.uint8), ry.contiguous().view(torch.uint8))
+        return
+    assert y_mx is None
+    if is_flex:
+        torch.testing.assert_close(actual.cpu(), ractual, rtol=1e-6, atol=1e-30)
+    if postprocess == "swiglu":
+        torch.testing.assert_close(y.cpu().float(), ry.float(), rtol=0.13 if is_flex else 2e-3, atol=1e-3)
+    else:
+        # the same float32 additions in the same order, the same casts: bit for bit
+        assert torch.equal(y.cpu().view(torch.uint8), ry.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("saturate", [False, True])
+@pytest.mark.parametrize("y_dtype", [torch.float8_e4m3fn, torch.float8_e5m2, torch.float16])
+def test_reduce_flex_output_saturation_and_global_scale(saturate, y_dtype, device):
+    """Sums far beyond the output type's range: clamped when saturating, the type's overflow value otherwise; the global
+    scale enters after the sum; the actual scale is the maximum before the division (flexpoint.py:137-188)."""
+    from triton_amd.numerics import OutFlexData
+    torch.manual_seed(1)
+    x = torch.randn(40, 6, 96) * 300
+    expected, gscale = torch.tensor([0.01]), torch.tensor([3.0])
+    actual = torch.zeros(1, device=device)
+    y, _ = reduce(x.to(device), dim=1, x_global_scale=gscale.to(device), y_dtype=y_dtype,
+                  y_flex=OutFlexData(expected_scale=expected.to(device), actual_scale=actual), y_flex_saturate_inf=saturate)
+    ry, _, ractual = MR.reduce_general_ref(x, 1, x_global_scale=gscale, y_dtype=y_dtype, y_expected_scale=expected,
+                                           y_saturate_inf=saturate)
+    a, b = y.cpu().float(), ry.float()
+    assert torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a), torch.nan_to_num(b))
+    torch.testing.assert_close(actual.cpu(), ractual, rtol=1e-6, atol=0)
+    if saturate:
+        assert torch.isfinite(a).all()
+
+
+def test_reduce_refuses_what_is_not_built(device):
+    from triton_amd.reduce import PostprocessFn
+    from triton_amd.specialize import FnSpecs
+    x = torch.randn(4, 3, 64, device=device)
+    with pytest.raises(NotImplementedError):
+        reduce(x, 1, postprocess_fn1=PostprocessFn(FnSpecs("gelu", None, (), reduction_n=1), ()))
+    with pytest.raises(NotImplementedError):
+        reduce(x, 1, unpadded_batch_size=torch.tensor([2], device=device))
+    with pytest.raises(NotImplementedError):
+        reduce(x, 1, y_value_pack_factor=2, y_has_mx=True)

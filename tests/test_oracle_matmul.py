@@ -174,3 +174,49 @@ def test_reduce_mx_small_integers_by_hand():
     for t in range(5):  # and that image is within half an fp8 step of the exact sum
         got = upcast_from_mxfp_ref(yv, ys, torch.float32, axis=-1)[t]
         assert torch.all((got - want[t]).abs() <= want[t].abs().reshape(2, 32).amax(dim=1).repeat_interleave(32) / 16 + 1e-6)
+
+
+def test_reduce_general_ref_hand_worked():
+    """Two rows, four columns, every optional operand, worked by hand (reduce.py:441-492, flexpoint.py:137-188)."""
+    x = torch.tensor([[[1.0, 2.0, 3.0, 4.0], [0.5, -1.0, 8.0, 2.0]]])            # [S0=1, R=2, S1=4]
+    mask = torch.tensor([[[1, 1, 1, 0], [1, 1, 0, 1]]], dtype=torch.bool)
+    scale = torch.tensor([[[2.0], [4.0]]])                                        # per reduced row
+    flex = torch.tensor([0.5])
+    # terms ((x * flex) * scale), masked: row 0 -> [1, 2, 3, 0], row 1 -> [1, -2, 0, 4]; sums [2, 0, 3, 4]
+    y, ymx, actual = MR.reduce_general_ref(x, 1, mask=mask, scale=scale, x_flex_scale=flex)
+    assert ymx is None and torch.equal(y, torch.tensor([[2.0, 0.0, 3.0, 4.0]]))
+    # plus_a with a = 10 over column pairs: (2 + 10) + (0 + 10) = 22, (3 + 10) + (4 + 10) = 27; global scale 2 -> 44, 54
+    y, _, actual = MR.reduce_general_ref(x, 1, mask=mask, scale=scale, x_flex_scale=flex, postprocess=("plus_a", 10.0),
+                                         x_global_scale=torch.tensor([2.0]), y_dtype=torch.float8_e4m3fn,
+                                         y_expected_scale=torch.tensor([0.125]), y_saturate_inf=True)
+    # actual scale is taken before the division: 54 / 448 + 1e-30; 44 / 0.125 = 352, 54 / 0.125 = 432 (both e4m3 numbers... 432
+    # lies between 416 and 448 on a grid of 32: ties to even -> 448)
+    assert abs(float(actual) - 54.0 / 448.0) < 1e-7
+    assert torch.equal(y.float(), torch.tensor([[352.0, 448.0]]))
+    # without saturation an overflowing value becomes NaN in float8_e4m3fn, with it the largest finite number
+    y_ns, _, _ = MR.reduce_general_ref(x, 1, y_dtype=torch.float8_e4m3fn, y_expected_scale=torch.tensor([0.001]))
+    y_s, _, _ = MR.reduce_general_ref(x, 1, y_dtype=torch.float8_e4m3fn, y_expected_scale=torch.tensor([0.001]), y_saturate_inf=True)
+    assert torch.isnan(y_ns.float()).all() and torch.equal(y_s.float(), torch.tensor([[448.0, 448.0, 448.0, 448.0]]))
+
+
+def test_reduce_general_ref_reduces_to_the_pinned_pieces():
+    """Without the extra operands it is reduce_ref; with SwiGLU it is swiglu_ref of the float32 sums; the microscaled
+    form is reduce_mx_ref; an fp8 input with a flex scale is the scaled sum of its exact float32 values."""
+    from oracle.mxfp_ref import downcast_to_mxfp_ref
+    torch.manual_seed(0)
+    x = torch.randn(5, 3, 64)
+    mask = torch.rand(5, 3, 1) > 0.3
+    scale = torch.rand(1, 3, 1) + 0.5
+    y, _, _ = MR.reduce_general_ref(x, 1, mask=mask, scale=scale)
+    assert torch.equal(y, MR.reduce_ref(x, 1, mask=mask, scale=scale))
+    y, _, _ = MR.reduce_general_ref(x, 1, postprocess=("swiglu", 1.702, 7.0))
+    assert torch.equal(y, MR.swiglu_ref(MR.reduce_ref(x, 1), 1.702, 7.0))
+    xv, xs = downcast_to_mxfp_ref(x, torch.float8_e4m3fn, axis=-1)
+    v, s2, _ = MR.reduce_general_ref(xv.contiguous(), 0, mask=mask, x_mxscale=xs.contiguous(), y_has_mx=True)
+    rv, rs = MR.reduce_mx_ref(xv.contiguous(), xs.contiguous(), 0, mask=mask)
+    assert torch.equal(v.view(torch.uint8), rv.view(torch.uint8)) and torch.equal(s2, rs)
+    x8 = (x / 2).to(torch.float8_e5m2)
+    y, _, actual = MR.reduce_general_ref(x8, 1, x_flex_scale=torch.tensor([2.0]), y_dtype=torch.float32)
+    want = (x8.float() * 2.0)[:, 0] + (x8.float() * 2.0)[:, 1] + (x8.float() * 2.0)[:, 2]
+    assert torch.equal(y, want)
+    assert abs(float(actual) - (float(want.abs().max()) / 3.4028234663852886e38 + 1e-30)) < 1e-36

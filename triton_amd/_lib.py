@@ -57,6 +57,24 @@ class MatmulArgs(C.Structure):
     ]
 
 
+class ReduceArgs(C.Structure):
+    """Mirror of `tamd_reduce_args`."""
+    _fields_ = [
+        ("x", C.c_void_p), ("x_dtype", C.c_int), ("S0", C.c_int64), ("R", C.c_int64), ("S1", C.c_int64),
+        ("xs0", C.c_int64), ("xsr", C.c_int64), ("xs1", C.c_int64),
+        ("x_mx_scale", C.c_void_p), ("xms0", C.c_int64), ("xmsr", C.c_int64), ("xms1", C.c_int64),
+        ("x_flex_scale", C.c_void_p), ("x_global_scale", C.c_void_p),
+        ("mask", C.c_void_p), ("ms0", C.c_int64), ("msr", C.c_int64), ("ms1", C.c_int64),
+        ("scale", C.c_void_p), ("ss0", C.c_int64), ("ssr", C.c_int64), ("ss1", C.c_int64),
+        ("postprocess", C.c_int), ("pp_arg0", C.c_float), ("pp_arg1", C.c_float), ("pp_has_arg1", C.c_int),
+        ("y", C.c_void_p), ("y_dtype", C.c_int), ("ys0", C.c_int64), ("ys1", C.c_int64),
+        ("y_expected_scale", C.c_void_p), ("y_actual_scale", C.c_void_p), ("y_saturate_inf", C.c_int),
+        ("y_mx_scale", C.c_void_p), ("yms0", C.c_int64), ("yms1", C.c_int64),
+    ]
+
+
+PP_NONE, PP_SWIGLU, PP_PLUS_A_PAIRSUM = 0, 1, 2
+
 _I64, _INT, _PTR, _F = C.c_int64, C.c_int, C.c_void_p, C.c_float
 _SIGNATURES = {
     "tamd_version": ([], C.c_int),
@@ -78,6 +96,7 @@ _SIGNATURES = {
     "tamd_matmul": ([C.POINTER(MatmulArgs), _PTR], C.c_int),
     "tamd_reduce": ([_PTR, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _PTR, _I64, _I64, _I64, _PTR, _I64, _I64, _I64,
                      _PTR, _INT, _I64, _I64, _PTR], C.c_int),
+    "tamd_reduce_ex": ([C.POINTER(ReduceArgs), _PTR], C.c_int),
     "tamd_swiglu": ([_PTR, _INT, _I64, _I64, _I64, _PTR, _I64, _F, _F, _INT, _PTR], C.c_int),
 }
 

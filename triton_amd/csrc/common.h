@@ -91,6 +91,8 @@ TAMD_DEVICE void store_from_f32(void *p, int64_t i, float v) {
   if constexpr (DT == TAMD_F16) ((uint16_t *)p)[i] = (uint16_t)f32_to_f16_bits(v);
 }
 
+__host__ __device__ inline bool is_fp8_type(int dt) { return dt == TAMD_FP8_E4M3 || dt == TAMD_FP8_E5M2; }
+
 inline int dtype_size(int dt) {
   switch (dt) {
     case TAMD_F32: return 4;

@@ -188,6 +188,206 @@ int launch_reduce(const void *x, int64_t S0, int64_t R, int64_t S1, int64_t xs0,
   return launch_status();
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The general reduction (reduce.py:375-492 of the reference, _reduce_forward_inner): every operand optional.
+//   t_r  = x[s0, r, c] (* 2^(e-127) of its 32-column group) * x_flex_scale * scale[s0, r, c], 0 where the mask is 0
+//   acc  = sum_r t_r                      float32, in index order
+//   o    = postprocess(acc)               none; SwiGLU of (gate, linear) column pairs; (pair + a) sums
+//   o   *= x_global_scale
+//   then either  flexpoint:  actual_scale <- max(actual_scale, max|o| / max_finite(y) + 1e-30); o /= expected_scale
+//                            (clamped to the finite range of y when saturating), cast to y's type
+//        or      MXFP8:      o /= expected_scale; per 32 output columns: scale = 2^ceil(log2(max|o| / 448)), values
+//                            o / scale as float8_e4m3fn (what tamd_downcast_mxfp makes of the same float32 numbers).
+// A thread owns PV consecutive input columns of one row s0 (PV = 8: vector loads when the layout allows; PV = RN: one
+// output per thread for narrow or strided inner axes).  The threads of a row are padded to a multiple of the threads
+// of a 32-column output group, so that a group's maximum is a shuffle over neighbouring lanes of one wave.
+// ---------------------------------------------------------------------------------------------------------------------
+TAMD_DEVICE float load_elem_f32(const void *p, int dt, int64_t i) {
+  switch (dt) {
+    case TAMD_F32: return ((const float *)p)[i];
+    case TAMD_BF16: return bf16_bits_to_f32(((const uint16_t *)p)[i]);
+    case TAMD_F16: return f16_bits_to_f32(((const uint16_t *)p)[i]);
+    case TAMD_FP8_E4M3: return __builtin_amdgcn_cvt_f32_fp8((int)((const uint8_t *)p)[i], 0);
+    default: return __builtin_amdgcn_cvt_f32_bf8((int)((const uint8_t *)p)[i], 0);
+  }
+}
+
+TAMD_DEVICE uint32_t narrow_bits(float v, int dt) {  // 8- or 16-bit output types
+  return dt == TAMD_BF16 ? (f32_to_bf16_bits(v) & 0xFFFFu) : (dt == TAMD_F16 ? (f32_to_f16_bits(v) & 0xFFFFu) : f32_to_fp8_bits(v, dt));
+}
+
+template <int PV, int RN>
+__global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int64_t threads_per_row, int vec_in, int vec_out) {
+  constexpr int NO = PV / RN;                         // outputs per thread
+  constexpr int TPG = 32 / NO > 0 ? 32 / NO : 1;      // threads of one 32-column output group
+  const int64_t S1 = a.S1, Y_S1 = S1 / RN;
+  const int64_t total = a.S0 * threads_per_row;
+  const int xsz = a.x_dtype == TAMD_F32 ? 4 : (is_fp8_type(a.x_dtype) ? 1 : 2);
+  const int ysz = a.y_dtype == TAMD_F32 ? 4 : (is_fp8_type(a.y_dtype) ? 1 : 2);
+  const float flex_in = a.x_flex_scale ? *a.x_flex_scale : 1.0f;
+  const float global = a.x_global_scale ? *a.x_global_scale : 1.0f;
+  const float inv_expected = a.y_expected_scale ? 1.0f / *a.y_expected_scale : 1.0f;
+  const float out_max = max_finite_of(a.y_dtype);
+  const bool clamp_out = a.y_expected_scale != nullptr && a.y_saturate_inf != 0 && a.y_mx_scale == nullptr;
+  uint32_t amax = 0;
+  for (int64_t base = (int64_t)blockIdx.x * 256; base < total; base += (int64_t)gridDim.x * 256) {
+    const int64_t i = base + threadIdx.x;
+    const bool live = i < total;
+    const int64_t s0 = live ? i / threads_per_row : 0;
+    const int64_t c0 = live ? (i - s0 * threads_per_row) * PV : S1;  // c0 >= S1: a padding thread of the row
+    float acc[PV];
+#pragma unroll
+    for (int j = 0; j < PV; ++j) acc[j] = 0.f;
+    if (c0 < S1) {
+      for (int64_t r = 0; r < a.R; ++r) {
+        float v[PV];
+        const int64_t xo = s0 * a.xs0 + r * a.xsr;
+        if (PV == 8 && vec_in) {  // unit inner stride, 8 columns inside S1, 8-element alignment of every row
+          if (xsz == 4) {
+            const float4 lo = *(const float4 *)((const float *)a.x + xo + c0), hi = *(const float4 *)((const float *)a.x + xo + c0 + 4);
+            v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4 % PV] = hi.x, v[5 % PV] = hi.y, v[6 % PV] = hi.z, v[7 % PV] = hi.w;
+          } else if (xsz == 2) {
+            const uint4 q = *(const uint4 *)((const uint16_t *)a.x + xo + c0);
+            const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int j = 0; j < PV / 2; ++j) {
+              v[2 * j] = a.x_dtype == TAMD_BF16 ? bf16_bits_to_f32(w[j] & 0xFFFFu) : f16_bits_to_f32(w[j] & 0xFFFFu);
+              v[2 * j + 1] = a.x_dtype == TAMD_BF16 ? bf16_bits_to_f32(w[j] >> 16) : f16_bits_to_f32(w[j] >> 16);
+            }
+          } else {
+            const uint2 q = *(const uint2 *)((const uint8_t *)a.x + xo + c0);
+#pragma unroll
+            for (int j = 0; j < PV; ++j) {
+              const int b = (int)(((j < 4 ? q.x : q.y) >> (8 * (j & 3))) & 0xFFu);
+              v[j] = a.x_dtype == TAMD_FP8_E4M3 ? __builtin_amdgcn_cvt_f32_fp8(b, 0) : __builtin_amdgcn_cvt_f32_bf8(b, 0);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < PV; ++j) v[j] = c0 + j < S1 ? load_elem_f32(a.x, a.x_dtype, xo + (c0 + j) * a.xs1) : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < PV; ++j) {
+          const int64_t c = c0 + j;
+          float t = v[j];
+          if (a.x_mx_scale) {
+            const uint32_t e = c < S1 ? a.x_mx_scale[s0 * a.xms0 + r * a.xmsr + (c / 32) * a.xms1] : 127u;
+            t *= bits_to_f32(e << 23);
+          }
+          t *= flex_in;
+          if (a.scale && c < S1) t *= a.scale[s0 * a.ss0 + r * a.ssr + c * a.ss1];
+          if (a.mask && c < S1 && !a.mask[s0 * a.ms0 + r * a.msr + c * a.ms1]) t = 0.f;
+          acc[j] += c < S1 ? t : 0.f;
+        }
+      }
+    }
+    // ---- post-processing over groups of RN columns
+    float o[NO];
+#pragma unroll
+    for (int j = 0; j < NO; ++j) {
+      if constexpr (RN == 1) o[j] = acc[j];
+      else if (a.postprocess == TAMD_PP_SWIGLU) o[j] = swiglu_f32(acc[2 * j], acc[2 * j + 1], a.pp_arg0, a.pp_arg1, a.pp_has_arg1 != 0);
+      else o[j] = (acc[2 * j] + a.pp_arg0) + (acc[2 * j + 1] + a.pp_arg0);
+      o[j] *= global;
+    }
+    const int64_t oc0 = c0 / RN;  // first output column
+    if (a.y_mx_scale) {
+      // MXFP8: the group's threads are TPG neighbouring lanes (rows are padded to whole groups of threads)
+      float m = 0.f;
+#pragma unroll
+      for (int j = 0; j < NO; ++j) {
+        o[j] *= inv_expected;
+        m = __builtin_fmaxf(m, oc0 + j < Y_S1 ? __builtin_fabsf(o[j]) : 0.f);
+      }
+#pragma unroll
+      for (int sh = TPG / 2; sh > 0; sh >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, sh));
+      const uint32_t sb = (f32_to_bits(m / 448.0f) + 0x007FFFFFu) & 0x7F800000u;
+      const float ds = bits_to_f32(sb);
+      const float qs = ds == 0.f ? 0.f : 1.0f / ds;
+#pragma unroll
+      for (int j = 0; j < NO; ++j) {
+        const float q = o[j] * qs;
+        o[j] = q != q ? q : __builtin_fminf(__builtin_fmaxf(q, -448.0f), 448.0f);
+      }
+      if (oc0 < Y_S1 && (threadIdx.x & (TPG - 1)) == 0) a.y_mx_scale[s0 * a.yms0 + (oc0 / 32) * a.yms1] = (uint8_t)(sb >> 23);
+    } else {
+      if (a.y_actual_scale) {
+#pragma unroll
+        for (int j = 0; j < NO; ++j)
+          if (oc0 + j < Y_S1) amax = absmax_bits(amax, o[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < NO; ++j) {
+        o[j] *= inv_expected;
+        if (clamp_out) o[j] = __builtin_fminf(__builtin_fmaxf(o[j], -out_max), out_max);
+      }
+    }
+    if (oc0 >= Y_S1) continue;
+    // ---- store: NO outputs, as one or two vector stores when the row is dense and aligned
+    if (NO > 1 && vec_out && oc0 + NO <= Y_S1) {
+      uint8_t *yp = (uint8_t *)a.y + (s0 * a.ys0 + oc0) * ysz;
+      if (ysz == 4) {
+#pragma unroll
+        for (int j = 0; j < NO; j += 4) *(float4 *)(yp + j * 4) = make_float4(o[j], o[(j + 1) % NO], o[(j + 2) % NO], o[(j + 3) % NO]);
+      } else if (ysz == 2) {
+        uint32_t w[NO / 2 > 0 ? NO / 2 : 1];
+#pragma unroll
+        for (int j = 0; j < NO / 2; ++j) w[j] = narrow_bits(o[2 * j], a.y_dtype) | (narrow_bits(o[2 * j + 1], a.y_dtype) << 16);
+        if constexpr (NO == 8) *(uint4 *)yp = make_uint4(w[0], w[1], w[2], w[3]);
+        else if constexpr (NO == 4) *(uint2 *)yp = make_uint2(w[0], w[1]);
+        else *(uint32_t *)yp = w[0];
+      } else {
+        uint32_t w[NO / 4 > 0 ? NO / 4 : 1];
+#pragma unroll
+        for (int j = 0; j < NO / 4; ++j)
+          w[j] = narrow_bits(o[4 * j], a.y_dtype) | (narrow_bits(o[4 * j + 1], a.y_dtype) << 8) |
+                 (narrow_bits(o[4 * j + 2], a.y_dtype) << 16) | (narrow_bits(o[4 * j + 3], a.y_dtype) << 24);
+        if constexpr (NO == 8) *(uint2 *)yp = make_uint2(w[0], w[1]);
+        else if constexpr (NO == 4) *(uint32_t *)yp = w[0];
+        else {
+#pragma unroll
+          for (int j = 0; j < NO; ++j) yp[j] = (uint8_t)narrow_bits(o[j], a.y_dtype);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NO; ++j) {
+        if (oc0 + j >= Y_S1) break;
+        const int64_t yi = s0 * a.ys0 + (oc0 + j) * a.ys1;
+        if (ysz == 4) ((float *)a.y)[yi] = o[j];
+        else if (ysz == 2) ((uint16_t *)a.y)[yi] = (uint16_t)narrow_bits(o[j], a.y_dtype);
+        else ((uint8_t *)a.y)[yi] = (uint8_t)narrow_bits(o[j], a.y_dtype);
+      }
+    }
+  }
+  if (a.y_actual_scale && !a.y_mx_scale) {
+    // wave maximum, then one atomic per wave; positive floats order like their bit patterns, NaN counts as +inf
+#pragma unroll
+    for (int sh = 32; sh > 0; sh >>= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)amax, sh);
+      amax = other > amax ? other : amax;
+    }
+    if (threadIdx.x % kWave == 0) {
+      amax = amax < 0x7F800000u ? amax : 0x7F800000u;
+      atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(__builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f)));
+    }
+  }
+}
+
+template <int PV, int RN>
+int launch_reduce_ex(const tamd_reduce_args &a, int vec_in, int vec_out, hipStream_t st) {
+  constexpr int NO = PV / RN;
+  constexpr int TPG = 32 / NO > 0 ? 32 / NO : 1;
+  int64_t tpr = (a.S1 + PV - 1) / PV;
+  if (a.y_mx_scale) tpr = (tpr + TPG - 1) / TPG * TPG;
+  const int64_t total = a.S0 * tpr;
+  int64_t blocks = (total + 255) / 256;
+  blocks = blocks > 65536 * 16 ? 65536 * 16 : (blocks < 1 ? 1 : blocks);
+  reduce_ex_kernel<PV, RN><<<dim3((unsigned)blocks), 256, 0, st>>>(a, tpr, vec_in, vec_out);
+  return launch_status();
+}
+
 }  // namespace tamd
 
 using namespace tamd;
@@ -252,4 +452,29 @@ extern "C" int tamd_swiglu(const void *a, int dtype, int64_t M, int64_t N_out, i
       return TAMD_E_INVALID;
   }
   return launch_status();
+}
+
+extern "C" int tamd_reduce_ex(const tamd_reduce_args *args, void *stream) {
+  if (!args) return TAMD_E_INVALID;
+  tamd_reduce_args a = *args;
+  if (a.S0 < 0 || a.R < 0 || a.S1 < 0) return TAMD_E_INVALID;
+  const int rn = a.postprocess == TAMD_PP_NONE ? 1 : 2;
+  if (a.postprocess != TAMD_PP_NONE && a.postprocess != TAMD_PP_SWIGLU && a.postprocess != TAMD_PP_PLUS_A_PAIRSUM) return TAMD_E_INVALID;
+  if (a.S1 % rn != 0) return TAMD_E_INVALID;
+  if (a.S0 == 0 || a.S1 == 0) return 0;
+  if (!a.y || (a.R > 0 && !a.x)) return TAMD_E_INVALID;
+  const bool x8 = is_fp8_type(a.x_dtype), y8 = is_fp8_type(a.y_dtype);
+  if (a.x_dtype != TAMD_F32 && a.x_dtype != TAMD_F16 && a.x_dtype != TAMD_BF16 && !x8) return TAMD_E_INVALID;
+  if (a.y_dtype != TAMD_F32 && a.y_dtype != TAMD_F16 && a.y_dtype != TAMD_BF16 && !y8) return TAMD_E_INVALID;
+  if (a.y_mx_scale && (a.y_dtype != TAMD_FP8_E4M3 || a.y_actual_scale)) return TAMD_E_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  const int xsz = a.x_dtype == TAMD_F32 ? 4 : (x8 ? 1 : 2), ysz = a.y_dtype == TAMD_F32 ? 4 : (y8 ? 1 : 2);
+  // eight columns per thread when the inner axis is dense, long enough and every row starts on an 8-element boundary
+  const bool wide = a.xs1 == 1 && a.S1 >= 64;
+  const int vec_in = wide && a.S1 % 8 == 0 && aligned(a.x, 8 * xsz) && a.xs0 % 8 == 0 && a.xsr % 8 == 0;
+  const int no = 8 / rn;
+  const int vec_out = wide && a.ys1 == 1 && (a.S1 / rn) % no == 0 && aligned(a.y, no * ysz < 16 ? no * ysz : 16) &&
+                      (a.ys0 * ysz) % (no * ysz < 16 ? no * ysz : 16) == 0;
+  if (wide) return rn == 1 ? launch_reduce_ex<8, 1>(a, vec_in, vec_out, st) : launch_reduce_ex<8, 2>(a, vec_in, vec_out, st);
+  return rn == 1 ? launch_reduce_ex<1, 1>(a, 0, 0, st) : launch_reduce_ex<2, 2>(a, 0, 0, st);
 }

@@ -339,15 +339,15 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         split_k = next((s for s in (8, 4, 2) if K % (s * 128) == 0 and K // s >= 1024), 1)
     if split_k > 1:
         flags = OptFlags(block_m=flags.block_m, split_k=split_k)
-        _matmul_split_k(args, flags.split_k, a, wd, b.dtype == FP4, out, fused_activation, act_alpha,
-                        limit if act == _lib.ACT_SWIGLU else None, bias)
+        _matmul_split_k(args, flags.split_k, a, wd, b.dtype == FP4, out, fused_activation, bias, flex.out_data,
+                        precision_config.flexpoint_saturate_inf)
         return finish()
     rc = _lib.lib().tamd_matmul(ctypes.byref(args), _lib.stream_ptr(a.device))
     _lib.check(rc, "matmul")
     return finish()
 
 
-def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, act_alpha, act_limit, bias):
+def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, bias, out_flex, saturate_inf):
     """K cut into `split_k` ranges (whole multiples of 128) whose float32 partial results [split_k, B, M, N] are
     summed afterwards (matmul.py:180-183, 471-472, 711-737 of the reference).  Every range applies the scales,
     betas, out_alpha and gammas (all linear), only the first adds the bias (_matmul.py:523-528), and the
@@ -357,11 +357,8 @@ def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, act_a
     (range s = batch entry s: activations, weights and scales advanced by s ranges, a bias that is zero for
     s > 0), so that they share the machine; anything else gets one launch per range."""
     from .reduce import reduce
-    from .swiglu import PrecisionConfig as SwigluPrecisionConfig, swiglu
     if args.scatter_indx or args.y_mx_scale:
         raise InapplicableConstraint("split_k cannot be combined with a scatter or a microscaled output")
-    if args.y_expected_scale or args.y_actual_scale or out.dtype.itemsize == 1:
-        raise InapplicableConstraint("split_k is built for 16- and 32-bit outputs without flexpoint scales")
     if args.w_mx_layout == _lib.SCALE_CDNA4:
         raise InapplicableConstraint("split_k needs weight scales in the strided layout")
     K, N = args.K, args.N
@@ -392,6 +389,7 @@ def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, act_a
         part.activation = _lib.ACT_NONE
         part.y, part.y_dtype = scratch.data_ptr(), _lib.F32
         part.y_stride_m, part.y_stride_z = scratch.stride(2), scratch.stride(0)
+        part.y_expected_scale = part.y_actual_scale = None
         part.force_variant = 0
         rc = _lib.lib().tamd_matmul(ctypes.byref(part), _lib.stream_ptr(out.device))
         _lib.check(rc, "matmul (split_k ranges as a batch)")
@@ -410,21 +408,19 @@ def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, act_a
         part.activation = _lib.ACT_NONE
         part.y, part.y_dtype = scratch[s].data_ptr(), _lib.F32
         part.y_stride_m, part.y_stride_z = scratch.stride(2), scratch.stride(1)
+        part.y_expected_scale = part.y_actual_scale = None
         rc = _lib.lib().tamd_matmul(ctypes.byref(part), _lib.stream_ptr(out.device))
         _lib.check(rc, "matmul (split_k range)")
+    # one finalising launch, as in the reference (matmul.py:711-737): sum of the partial results, the fused activation
+    # as the reduction's post-processing function, the output's flexpoint scales, the cast
+    from .reduce import PostprocessFn
     parts = scratch.view(n_split, batch * rows, N)
-    direct = out.is_contiguous() and fused_activation.specs.name == "dflt"
-    if direct:
-        reduce(parts, dim=0, y=out.view(batch * rows, N), y_dtype=out.dtype)
-        return
-    total, _ = reduce(parts, dim=0, y_dtype=torch.float32)
-    if fused_activation.specs.name == "swiglu":
-        total = swiglu(total, act_alpha, SwigluPrecisionConfig(act_limit))
-    if out.is_contiguous():
-        # float32 -> output type with the library's own kernel: a sum over an axis of length one
-        reduce(total[None], dim=0, y=out.view(batch * rows, -1), y_dtype=out.dtype)
-    else:
-        out.copy_(total.view(out.shape))
+    pp = PostprocessFn(fused_activation.specs, fused_activation.fn_args) if fused_activation.specs.name != "dflt" else None
+    dst = out if out.is_contiguous() else torch.empty(out.shape, dtype=out.dtype, device=out.device)
+    reduce(parts, dim=0, y=dst.view(batch * rows, -1), y_dtype=out.dtype, y_flex=out_flex, y_flex_saturate_inf=saturate_inf,
+           postprocess_fn1=pp)
+    if dst is not out:
+        out.copy_(dst)
 
 
 matmul_ogs = matmul
