@@ -48,6 +48,11 @@ WORKLOADS = {
     # quantise / dequantise of weights in the matmul's layout: [8, 2880, 5760] float32 -> MXFP4 along K -> bfloat16
     "quant": dict(E=8, K=2880, N=5760, quant=True),
     "dequant": dict(E=8, K=2880, N=5760, dequant=True),
+    # the whole MoE layer as the reference's bench/bench_mlp.py:60-96 runs it on one GPU, at the largest point of its
+    # sweep (:256-279: d_model 5760, 128 experts, top-4, 64 rows per expert -> 2048 tokens, fp8 activations, MXFP4
+    # weights): gate matmul -> top-k + softmax -> metadata -> FC1 + SwiGLU (gathered rows) -> FC2 (rows scattered back
+    # to token order) -> sum over the k slots
+    "mlp": dict(bpe=64, dim1=5760, dim2=5760, E=128, k=4, mlp=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
     # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
     "hbm_copy": dict(bytes=1 << 30),
@@ -555,6 +560,128 @@ def run_fc1(args, cfg, name):
     return out
 
 
+def run_mlp(args, cfg, name):
+    """bench/bench_mlp.py:60-96 of the reference with one rank: every stage is timed with HIP events, and checked
+    against the oracle given the GPU's own output of the stage before (logits -> routing, bit-exact; FC1 and FC2 on a
+    sample of experts, within the fp8 output step; the combine, bit-exact)."""
+    from oracle import matmul_ref as MR
+    from oracle import routing_ref as RR
+    from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
+    from triton_amd.reduce import reduce
+    from triton_amd.routing import routing
+    from triton_amd.swiglu import swiglu_fn
+    from triton_amd.numerics_details.mxfp import downcast_to_mxfp
+    E, k, d1, d2 = cfg["E"], cfg["k"], cfg["dim1"], cfg["dim2"]
+    T = cfg["bpe"] * E // k
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    rnd = lambda *shape: torch.randn(shape, generator=g, device=dev, dtype=torch.float32)
+    wg = rnd(d1, E).to(torch.bfloat16).t().contiguous().t()  # [d1, E] with unit stride along K, as quantize_weight leaves it
+    bg, b1, b2 = rnd(E), rnd(E, d2), rnd(E, d1)
+
+    def quantise(K, N):
+        from triton_amd.tensor import FP4, empty
+        from triton_amd.tensor_details.dtype import UINT8
+        from triton_amd.tensor_details.layout import StridedLayout
+        vals = empty((E, K, N), FP4, dev, StridedLayout(-2)).storage.data
+        scales = empty((E, K // 32, N), UINT8, dev, StridedLayout(-2)).storage.data
+        for e in range(E):
+            v, sc = downcast_to_mxfp(rnd(1, K, N).to(torch.bfloat16), torch.uint8, axis=1)
+            vals[e].copy_(v[0])
+            scales[e].copy_(sc[0])
+        return vals, scales
+    w1, s1 = quantise(d1, d2)
+    w2, s2 = quantise(d2 // 2, d1)
+    x8 = rnd(T, d1).to(torch.float8_e4m3fn)
+    x16 = x8.to(torch.bfloat16)
+    pc1 = PrecisionConfig(b_mx_scale=scales_for_matmul(s1, args.scale_layout), b_microblock_size=32)
+    pc2 = PrecisionConfig(b_mx_scale=scales_for_matmul(s2, args.scale_layout), b_microblock_size=32)
+    act1 = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.0, 1.0))
+    names = ("gate_matmul", "routing", "fc1_swiglu", "fc2_scatter", "combine")
+
+    def step(ev=None):
+        mark = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
+        mark(0)
+        logits = matmul(x16, wg, bg)
+        mark(1)
+        r = routing(logits, k)
+        mark(2)
+        y1 = matmul(x8, w1, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
+        mark(3)
+        y2 = matmul(y1, w2, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
+        mark(4)
+        z, _ = reduce(y2.view(T, k, d1), dim=1)
+        mark(5)
+        return logits, r, y1, y2, z
+
+    spin_up(step)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        logits, r, y1, y2, z = step(events[i])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    stage_ms = {n: sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i, n in enumerate(names)}
+    rows = T * k
+    flops = {"gate_matmul": 2.0 * T * d1 * E, "fc1_swiglu": 2.0 * rows * d1 * d2, "fc2_scatter": 2.0 * rows * (d2 // 2) * d1}
+    n_active = int((r.col_sum > 0).sum())
+    w_bytes = lambda K, N: n_active * (K // 2 * N + K // 32 * N + N * 4)
+    bytes_ = {"gate_matmul": T * d1 * 2 + d1 * E * 2 + T * E * 2, "fc1_swiglu": rows * d1 + w_bytes(d1, d2) + rows * d2 // 2,
+              "fc2_scatter": rows * d2 // 2 + w_bytes(d2 // 2, d1) + rows * d1, "combine": rows * d1 + T * d1}
+    stages = {}
+    for n in names:
+        st = {"ms": round(stage_ms[n], 4)}
+        if n in flops:
+            st["tflops"] = round(flops[n] / (stage_ms[n] * 1e-3) / 1e12, 1)
+        if n in bytes_:
+            st["algorithmic_gbs"] = round(bytes_[n] / (stage_ms[n] * 1e-3) / 1e9, 1)
+        stages[n] = st
+    # ---- parity, stage by stage, each against the oracle fed with the GPU's output of the stage before
+    logits_ref = MR.matmul_ref(x16.cpu(), wg.cpu(), bg.cpu())
+    logits_ok = bool(torch.allclose(logits.cpu().float(), logits_ref.float(), rtol=2e-2, atol=2e-1))
+    ref = RR.routing_ref(logits.cpu(), k)
+    routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(r.col_sum.cpu(), ref["col_sum"])
+                      and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]))
+    n_e = 2 if args.cpu_experts <= 0 else min(args.cpu_experts, E)
+    sizes = ref["col_sum"][:n_e]
+    n_rows = int(sizes.sum())
+    t0 = time.perf_counter()
+    y1_ref = MR.matmul_ref(x8.cpu(), w1[:n_e].cpu(), b1[:n_e].cpu(), slice_sizes=sizes, gather_indx=ref["gather_indx"][:n_rows],
+                           b_mx_scale=s1[:n_e].cpu(), fused_swiglu=(1.0, 1.0))
+    y2_ref = MR.matmul_ref(y1[:n_rows].cpu(), w2[:n_e].cpu(), b2[:n_e].cpu(), slice_sizes=sizes, b_mx_scale=s2[:n_e].cpu())
+    cpu_s = time.perf_counter() - t0
+    # fp8 outputs: one step of the type (2^-3 relative) where an fp32 sum lands on a rounding boundary
+    fc1_ok = bool(torch.allclose(y1[:n_rows].cpu().float(), y1_ref.float(), rtol=0.13, atol=2e-2))
+    got2 = y2.cpu()[ref["scatter_indx"][:n_rows].long()].float()
+    fc2_ok = bool(torch.allclose(torch.nan_to_num(got2, nan=1e30), torch.nan_to_num(y2_ref.float(), nan=1e30), rtol=0.13, atol=1.0))
+    z_ref, _, _ = MR.reduce_general_ref(y2.view(T, k, d1)[:256].cpu(), 1)
+    a, b = z[:256].cpu().float(), z_ref.float()
+    combine_ok = bool(torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a), torch.nan_to_num(b)))
+    mm_ms = stage_ms["fc1_swiglu"] + stage_ms["fc2_scatter"]
+    mm_flops = flops["fc1_swiglu"] + flops["fc2_scatter"]
+    tflops = mm_flops / (mm_ms * 1e-3) / 1e12
+    out = base_line(args, "moe_mlp_tokens_per_s", round(T / (ms_per_step * 1e-3), 1), "tokens/s", ms_per_step,
+                    "fp8e4m3 x mxfp4 (fp32 accumulate), bf16 gate",
+                    f"{name}: gate matmul + routing + FC1/SwiGLU + FC2 + combine, tokens={T}, d_model={d1}, experts={E}, "
+                    f"top-{k}, W1 mxfp4 [{E},{d1},{d2}], W2 mxfp4 [{E},{d2 // 2},{d1}]", scale_layout=args.scale_layout)
+    out["stages"] = stages
+    out["roofline"] = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                       "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": None, "kernel": "mm_x8_mxfp4_kernel (FC1 + FC2)",
+                       "kernel_ms": round(mm_ms, 4), "algorithmic_flops": mm_flops,
+                       "algorithmic_bytes": bytes_["fc1_swiglu"] + bytes_["fc2_scatter"],
+                       "hbm_gbs": round((bytes_["fc1_swiglu"] + bytes_["fc2_scatter"]) / (mm_ms * 1e-3) / 1e9, 1)}
+    out["cpu_baseline"] = {"value": round((2.0 * n_rows * d1 * d2 + 2.0 * n_rows * (d2 // 2) * d1) / cpu_s / 1e12, 5),
+                           "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                           "sample": f"oracle FC1 + FC2 on the first {n_e} of {E} experts ({n_rows} of {rows} rows), {cpu_s:.1f} s"}
+    out["parity"] = {"gate_logits_within_2e-2": logits_ok, "routing_bit_exact": routing_ok, "fc1_sample_within_fp8_step": fc1_ok,
+                     "fc2_sample_within_fp8_step": fc2_ok, "combine_bit_exact": combine_ok}
+    return out
+
+
 def run_workload(args, name):
     cfg = WORKLOADS[name]
     if name == "hbm_copy":
@@ -567,6 +694,8 @@ def run_workload(args, name):
         return run_quant(args, cfg, name)
     if cfg.get("fc2"):
         return run_fc2(args, cfg, name)
+    if cfg.get("mlp"):
+        return run_mlp(args, cfg, name)
     return run_fc1(args, cfg, name)
 
 

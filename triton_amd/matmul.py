@@ -366,7 +366,8 @@ def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, bias,
         # the kernel for 16-bit weights bounds its K tail by the end of the expert's weights, which a range
         # that starts inside them would move
         raise InapplicableConstraint("split_k with 16-bit weights needs K to be a multiple of 64")
-    chunk = -(-(-(-K // split_k)) // 128) * 128
+    align = 128 if w_is_fp4 else 64  # whole stages of the kernel that runs the ranges
+    chunk = -(-(-(-K // split_k)) // align) * align
     n_split = -(-K // chunk)
     batch, rows = out.shape[0], out.shape[1]
     scratch = torch.empty((n_split, batch, rows, N), dtype=torch.float32, device=out.device)
