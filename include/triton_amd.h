@@ -145,6 +145,18 @@ int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_t n_indx, i
                           int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream);
 
 /*
+ * The whole routing step in one call: tamd_topk_forward (softmax over the k picked, indices chosen here) followed by
+ * tamd_routing_metadata on its indices -- the composition of tests/test_distributed.py:201-208 as one entry point,
+ * so that a binding pays for one foreign call per batch.  Arguments as in the two functions; y_indx is [n_rows, k]
+ * with unit stride along k.
+ */
+int tamd_routing(const void *logits, int dtype, int64_t stride, int n_rows, int n_cols, int k, void *y_vals,
+                 int16_t *y_indx, uint32_t *bits, int64_t bits_stride_row, int64_t bits_stride_word, int32_t *col_sum,
+                 int32_t *col_sorted_indx, int32_t *row_sorted_indx, int32_t *gather_indx, int32_t *offs,
+                 int64_t offs_pitch, int32_t *schedule, int64_t sched_pitch, int max_n_blocks, int32_t *workspace,
+                 void *stream);
+
+/*
  * tamd_routing_metadata for callers that cannot allocate (code under HIP graph capture, serving loops and
  * harnesses that forbid hipMalloc).  No counterpart in the reference, where every workspace is a torch allocation
  * made per call.  Same arguments and results as tamd_routing_metadata without `workspace`: the intermediate

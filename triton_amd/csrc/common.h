@@ -3,6 +3,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
+#include <unordered_set>
+
 #include "../../include/triton_amd.h"
 
 #define TAMD_DEVICE __device__ __forceinline__
@@ -106,6 +110,46 @@ inline int dtype_size(int dt) {
 }
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// One-time set-up per kernel and device, kept out of the per-call path: raising a kernel's dynamic LDS limit (an
+// attribute of the function in the device's loaded code object) and the device's CU count.  The only process-wide
+// state of the library besides its code objects; values never change once set, so calls stay re-entrant.
+inline int current_device(int &dev) {
+  hipError_t e = hipGetDevice(&dev);
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+inline int raise_lds_limit_once(const void *kern) {
+  static std::mutex mu;
+  static std::unordered_set<uint64_t> done;
+  int dev = 0;
+  if (int rc = current_device(dev)) return rc;
+  const uint64_t key = ((uint64_t)(uint32_t)dev << 48) ^ (uint64_t)(uintptr_t)kern;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count(key)) return 0;
+  }
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e != hipSuccess) return (int)e;
+  std::lock_guard<std::mutex> lock(mu);
+  done.insert(key);
+  return 0;
+}
+
+inline int cu_count(int &cus) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> cached[kMaxDevices];
+  int dev = 0;
+  if (int rc = current_device(dev)) return rc;
+  if (dev >= 0 && dev < kMaxDevices) {
+    cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus > 0) return 0;
+  }
+  hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev >= 0 && dev < kMaxDevices) cached[dev].store(cus, std::memory_order_relaxed);
+  return 0;
+}
 
 inline int launch_status() {
   hipError_t e = hipGetLastError();

@@ -177,8 +177,7 @@ int launch_w16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int64_t launch = ((total + 7) / 8) * 8;
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
   auto kern = mm_x16_w16_kernel<XDT, BM, ACT, WKC>;
-  hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e != hipSuccess) return (int)e;
+  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
   kern<<<dim3((unsigned)launch), 256, PIPE > OUT_BYTES ? PIPE : OUT_BYTES, st>>>(a, grid_n, total);
   return launch_status();
 }

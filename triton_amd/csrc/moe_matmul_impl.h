@@ -820,9 +820,7 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
     kern = sc_in_lds ? mm_x8_mxfp4_kernel<XDT, BM, ACT, true> : mm_x8_mxfp4_kernel<XDT, BM, ACT, false>;
   else
     kern = sc_in_lds ? mm_x16_mxfp4_kernel<XDT, BM, ACT, true> : mm_x16_mxfp4_kernel<XDT, BM, ACT, false>;
-  // raising the dynamic LDS limit is idempotent, so doing it on every launch keeps the entry point stateless
-  hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e != hipSuccess) return (int)e;
+  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
   // row blocks walked together: as many as one expert (or batch entry) has, while their activation
   // rows (BM x K each) fit comfortably in one XCD's 4 MB L2
   const int64_t rows_per_slice = a.block_schedule ? a.M / a.n_experts : a.M;

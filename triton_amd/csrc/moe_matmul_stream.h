@@ -477,14 +477,11 @@ int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int n_cg = (a.N + 15) / 16;
   const int64_t upper = (int64_t)grid_m * n_cg;
   if (upper <= 0) return 0;
-  int dev = 0, cus = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  if (e != hipSuccess) return (int)e;
+  int cus = 0;
+  if (int rc = cu_count(cus)) return rc;
   const int wgs = (int)(upper < cus ? upper : cus);
   auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, A8>;
-  e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e != hipSuccess) return (int)e;
+  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
   kern<<<dim3((unsigned)wgs), 512, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
   return launch_status();
 }

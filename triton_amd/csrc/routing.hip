@@ -597,8 +597,7 @@ static int ragged_launch(const int32_t *slice_sizes, int n_slices, int32_t *offs
                          int32_t *schedule, int64_t sched_pitch, int max_n_blocks, hipStream_t st) {
   const size_t lds = 6 * (size_t)(n_slices + 1) * 4;
   if (lds > 150 * 1024) return TAMD_E_UNSUPPORTED;  // more than ~6000 slices
-  hipError_t e = hipFuncSetAttribute((const void *)ragged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-  if (e != hipSuccess) return (int)e;
+  if (int rc = raise_lds_limit_once((const void *)ragged_kernel)) return rc;
   int64_t wgs = (5 * (int64_t)max_n_blocks + 4095) / 4096;  // about four entries per thread
   wgs = wgs < 1 ? 1 : (wgs > 256 ? 256 : wgs);
   ragged_kernel<<<dim3((unsigned)wgs), 1024, lds, st>>>(slice_sizes, n_slices, offs, offs_pitch, schedule, sched_pitch,
@@ -651,8 +650,7 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
     if (NC <= 64 && ints * 4 <= 156 * 1024) {  // beyond ~4096 entries one CU is slower than three launches
       int nbits = 0;
       while ((1 << nbits) < n_cols) ++nbits;
-      hipError_t e = hipFuncSetAttribute((const void *)meta_fused_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-      if (e != hipSuccess) return (int)e;
+      if (int rc = raise_lds_limit_once((const void *)meta_fused_kernel)) return rc;
       meta_fused_kernel<<<1, 1024, (size_t)ints * 4, (hipStream_t)stream>>>(
           indx, indx_is_int16, (int)n_indx, n_cols, k, nbits, (int)NC, (int)P, col_sum, col_sorted_indx, row_sorted_indx,
           gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
@@ -666,8 +664,7 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
     MetaPlan p = make_meta_plan(n_indx, n_cols);
     hist_kernel<<<dim3((unsigned)p.n_blocks), 256, (size_t)p.CH * n_cols * 4, st>>>(
         indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, workspace + p.off_chunk_pref, workspace + p.off_block_tot);
-    hipError_t e = hipFuncSetAttribute((const void *)scan_ragged_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return (int)e;
+    if (int rc = raise_lds_limit_once((const void *)scan_ragged_kernel)) return rc;
     int64_t wgs = (5 * (int64_t)max_n_blocks + 4095) / 4096;
     wgs = wgs < 1 ? 1 : (wgs > 64 ? 64 : wgs);
     scan_ragged_kernel<<<dim3((unsigned)wgs), 1024, sr_lds, st>>>(
@@ -688,6 +685,18 @@ extern "C" int tamd_routing_metadata(const void *indx, int indx_is_int16, int64_
                                      int32_t *gather_indx, int32_t *offs, int64_t offs_pitch, int32_t *schedule,
                                      int64_t sched_pitch, int max_n_blocks, int32_t *workspace, void *stream) {
   return routing_metadata_impl(indx, indx_is_int16, n_indx, n_cols, k, col_sum, col_sorted_indx, row_sorted_indx,
+                               gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, workspace, stream);
+}
+
+extern "C" int tamd_routing(const void *logits, int dtype, int64_t stride, int n_rows, int n_cols, int k, void *y_vals,
+                            int16_t *y_indx, uint32_t *bits, int64_t bits_stride_row, int64_t bits_stride_word,
+                            int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx, int32_t *gather_indx,
+                            int32_t *offs, int64_t offs_pitch, int32_t *schedule, int64_t sched_pitch, int max_n_blocks,
+                            int32_t *workspace, void *stream) {
+  const int rc = tamd_topk_forward(logits, dtype, stride, n_rows, n_cols, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row,
+                                   bits_stride_word, stream);
+  if (rc != 0) return rc;
+  return routing_metadata_impl(y_indx, 1, (int64_t)n_rows * k, n_cols, k, col_sum, col_sorted_indx, row_sorted_indx,
                                gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, workspace, stream);
 }
 

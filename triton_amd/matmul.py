@@ -69,6 +69,13 @@ class PrecisionConfig:
     enforce_bitwise_invariance: bool = False
 
 
+# what `matmul` uses for arguments left out; never written to (c_microblock_size is only filled in for a caller's
+# own config with c_mx_scale)
+_DEFAULT_PRECISION = PrecisionConfig()
+_DEFAULT_ACTIVATION = FusedActivation(FnSpecs.default(), tuple())
+_DEFAULT_EPILOGUE = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+
+
 def _data(t):
     return t.storage.data if isinstance(t, Tensor) else t
 
@@ -91,11 +98,11 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     gather_indx / scatter_indx: int32 row maps (scatter -1 drops the row).
     """
     if precision_config is None:
-        precision_config = PrecisionConfig()
+        precision_config = _DEFAULT_PRECISION
     if fused_activation is None:
-        fused_activation = FusedActivation(FnSpecs.default(), tuple())
+        fused_activation = _DEFAULT_ACTIVATION
     if epilogue is None:
-        epilogue = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
+        epilogue = _DEFAULT_EPILOGUE
     is_input_batched = a.ndim == 3
     if is_input_batched:
         assert gather_indx is None, "gather not supported in batched mode"
@@ -146,8 +153,13 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
             raise NotImplementedError("per-batch flexpoint output scales are not built (one float32 value expected)")
     # ---- weights
     b_scale = precision_config.b_mx_scale
-    if not isinstance(b, Tensor):
-        b = wrap_torch_tensor(b, dtype=FP4 if b.dtype == torch.uint8 else None)
+    # weights: storage tensor, whether they are packed e2m1 codes, logical shape (a packed axis counts twice)
+    if isinstance(b, Tensor):
+        b_data, b_fp4, b_shape = b.storage.data, b.dtype == FP4, list(b.shape)
+    else:
+        b_data, b_fp4, b_shape = b, b.dtype == torch.uint8, list(b.shape)
+        if b_fp4:
+            b_shape[b.stride().index(1)] *= 2
     if b_scale is not None:
         assert precision_config.b_microblock_size is not None, \
             "precision_config.b_microblock_size is required when precision_config.b_mx_scale is set"
@@ -158,27 +170,28 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         assert b_scale.dtype == torch.uint8, f"Unsupported microscale dtype {b_scale.dtype}"
     if isinstance(a, Tensor):
         a = a.storage.data
-    if b_scale is not None and b.dtype != FP4:
+    if b_scale is not None and not b_fp4:
         # MXFP8 weights: dequantised to bfloat16 by the library's upcast kernel, as the reference's torch path does
         # (matmul.py:788-794), and multiplied by the kernel for unquantised weights
-        w8 = b.storage.data
+        w8 = b_data
         if w8.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2) or b_scale_cdna4:
             raise NotImplementedError("microscaled weights are built as MXFP4, or MXFP8 with scales in the strided layout")
         if a.dtype != torch.bfloat16 or a_mx_scale is not None:
             raise NotImplementedError("MXFP8 weights are built for bfloat16 activations")
         from .numerics_details.mxfp import upcast_from_mxfp
-        b = wrap_torch_tensor(upcast_from_mxfp(w8, b_scale, torch.bfloat16, axis=-2))
+        b_data = upcast_from_mxfp(w8, b_scale, torch.bfloat16, axis=-2)
+        b_shape = list(b_data.shape)
         b_scale = None
     a = flex.lhs_data.reinterpret(a)
-    w = flex.rhs_data.reinterpret(b.storage.data)
+    w = flex.rhs_data.reinterpret(b_data)
     a_dtype = a.dtype  # the type the output defaults to
     fp8_types = (torch.float8_e4m3fn, torch.float8_e5m2)
-    if b.dtype != FP4 and w.dtype in fp8_types and a.dtype in fp8_types and a_mx_scale is None:
+    if not b_fp4 and w.dtype in fp8_types and a.dtype in fp8_types and a_mx_scale is None:
         # fp8 x fp8 with per-tensor scales (tests/test_matmul.py:150-154 of the reference): every fp8 number is a
         # bfloat16 number, so both operands are widened (exactly) and multiplied by the kernel for 16-bit weights; the
         # flex scales enter in its epilogue as they do for any other pair of types
         a, w = a.to(torch.bfloat16), w.to(torch.bfloat16)
-    if b.dtype != FP4 and w.stride(-1) == 1 and (w.shape[-1] * w.element_size()) % 16 != 0 \
+    if not b_fp4 and w.stride(-1) == 1 and (w.shape[-1] * w.element_size()) % 16 != 0 \
             and (w.shape[-2] * w.element_size()) % 16 == 0:
         # unquantised weights with unit stride along N whose rows do not start on 16-byte boundaries: the kernel copies
         # 16 bytes at a time, so they are laid out with unit stride along K instead (same values)
@@ -188,14 +201,14 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     assert a.stride(-1) == 1 or a.shape[-1] == 1, "a must be contiguous along K"
     # ---- shapes
     K = a.shape[-1]
-    K_W, N = b.shape[-2:]
+    K_W, N = b_shape[-2:]
     assert K == K_W, f"inner dimensions differ: {K} vs {K_W}"
     ragged = a_ragged_metadata is not None
     M = a.shape[-2] if gather_indx is None else gather_indx.shape[0]
     if ragged:
         n_slices, batch = a_ragged_metadata.n_slices, 1
-    elif b.ndim == 3:
-        n_slices = batch = b.shape[0]
+    elif len(b_shape) == 3:
+        n_slices = batch = b_shape[0]
     else:
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
@@ -243,7 +256,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     # ---- tile choice
     flags = make_opt_flags(M, N, K, n_slices, ragged,
                            a_ragged_metadata.expected_slice_size if ragged else None)
-    args = _lib.MatmulArgs()
+    args = _lib.MatmulArgBag()
     args.x, args.x_dtype = a.data_ptr(), _lib.dtype_code(a.dtype)
     args.x_stride_m = a.stride(-2)
     args.x_stride_z = a.stride(0) if a.ndim == 3 else 0
@@ -257,7 +270,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         args.x_mx_stride_z = a_mx_scale.stride(0) if a_mx_scale.ndim == 3 else 0
     wd = w if w.ndim == 3 else w[None]
     args.w = wd.data_ptr()
-    if b.dtype == FP4:
+    if b_fp4:
         assert b_scale is not None, "MXFP4 weights need precision_config.b_mx_scale"
         args.w_dtype = _lib.MXFP4
         want = [wd.shape[0], K // MXFP_BLOCK_SIZE, N]
@@ -339,10 +352,10 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         split_k = next((s for s in (8, 4, 2) if K % (s * 128) == 0 and K // s >= 1024), 1)
     if split_k > 1:
         flags = OptFlags(block_m=flags.block_m, split_k=split_k)
-        _matmul_split_k(args, flags.split_k, a, wd, b.dtype == FP4, out, fused_activation, bias, flex.out_data,
+        _matmul_split_k(args.pack(), flags.split_k, a, wd, b_fp4, out, fused_activation, bias, flex.out_data,
                         precision_config.flexpoint_saturate_inf)
         return finish()
-    rc = _lib.lib().tamd_matmul(ctypes.byref(args), _lib.stream_ptr(a.device))
+    rc = _lib.lib().tamd_matmul(ctypes.byref(args.pack()), _lib.stream_ptr(a.device))
     _lib.check(rc, "matmul")
     return finish()
 
