@@ -273,7 +273,7 @@ def run_quant(args, cfg, name):
         rv, rs = downcast_to_mxfp_ref(sample, torch.uint8, 1)
         cpu_s = time.perf_counter() - t0
         ok = bool(torch.equal(v[:1, :, :256].cpu(), rv) and torch.equal(s[:1, :, :256].cpu(), rs))
-        what, kern, dtype = "downcast_to_mxfp: float32 -> e2m1 codes + e8m0 scales", "downcast_cols_kernel", "f32 -> mxfp4"
+        what, kern, dtype = "downcast_to_mxfp: float32 -> e2m1 codes + e8m0 scales", "downcast_cols_tile_kernel", "f32 -> mxfp4"
         parity = {"codes_and_scales_bit_exact": ok}
     else:
         v, s = downcast_to_mxfp(w, torch.uint8, axis=1)
@@ -284,7 +284,7 @@ def run_quant(args, cfg, name):
         ref = upcast_from_mxfp_ref(vs, ss, torch.bfloat16, 1)
         cpu_s = time.perf_counter() - t0
         ok = bool(torch.equal(y[:1, :, :256].cpu().view(torch.int16), ref.view(torch.int16)))
-        what, kern, dtype = "upcast_from_mxfp: e2m1 codes + e8m0 scales -> bfloat16", "upcast_cols_kernel", "mxfp4 -> bf16"
+        what, kern, dtype = "upcast_from_mxfp: e2m1 codes + e8m0 scales -> bfloat16", "upcast_cols_tile_kernel", "mxfp4 -> bf16"
         parity = {"values_bit_exact": ok}
     gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     out = base_line(args, "mxfp_gbs", round(alg_bytes / (wall * 1e-3) / 1e9, 1), "GB/s", wall, dtype,

@@ -1,11 +1,13 @@
 // MXFP4 / MXFP8 quantise / dequantise for gfx950.  Bandwidth kernels: 128-bit global
 // accesses, one 32-element group handled by 4 lanes (quantised axis contiguous)
-// or by one lane per column (quantised axis strided, i.e. the weight layout).
+// or by one lane per column set (quantised axis strided, i.e. the weight layout: tiles
+// of 16 or 32 groups x 128 or 256 columns that pass through LDS).
 //
 // Arithmetic follows numerics_details/mxfp.py:212-363 and :384-449 of the
 // reference: scale = 2^ceil(log2(max/6)) taken from the float32 bit pattern,
 // q = x * (1/scale), round-to-nearest-even onto {0,.5,1,1.5,2,3,4,6}, saturate.
 #include "common.h"
+#include <type_traits>
 
 namespace tamd {
 
@@ -17,6 +19,33 @@ TAMD_DEVICE uint32_t e2m1_pair(float q0, float q1) {
   if (q0 != q0) c = (c & 0xF0u) | 7u | ((f32_to_bits(q0) >> 28) & 8u);
   if (q1 != q1) c = (c & 0x0Fu) | ((7u | ((f32_to_bits(q1) >> 28) & 8u)) << 4);
   return c;
+}
+
+// The same conversion with the division by the group's scale (a power of two, `ds`) done by the instruction:
+// writes the code pair of (a / ds, b / ds) into byte BS of `old`.  Exact wherever a / ds is: callers keep to
+// scales whose reciprocal is a normal float and to groups without NaN.
+template <int BS>
+TAMD_DEVICE uint32_t e2m1_pair_scaled(uint32_t old, float a, float b, float ds) {
+  return (uint32_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, ds, BS);
+}
+// 8 e2m1 codes of one column (rows l0 .. l0+7, v[i] = row l0 + i) -> one 32-bit word
+TAMD_DEVICE uint32_t e2m1_word_scaled(const float (&v)[8], float ds) {
+  uint32_t w = 0;
+  w = e2m1_pair_scaled<0>(w, v[0], v[1], ds);
+  w = e2m1_pair_scaled<1>(w, v[2], v[3], ds);
+  w = e2m1_pair_scaled<2>(w, v[4], v[5], ds);
+  w = e2m1_pair_scaled<3>(w, v[6], v[7], ds);
+  return w;
+}
+
+// 16-byte accesses to memory that is touched once (non-temporal)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+TAMD_DEVICE uint4 load_once(const void *p) {
+  u32x4_t q = __builtin_nontemporal_load((const u32x4_t *)p);
+  return make_uint4(q.x, q.y, q.z, q.w);
+}
+TAMD_DEVICE void store_once(void *p, uint4 v) {
+  __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, (u32x4_t *)p);
 }
 
 // Value kinds of a microscaled tensor: e2m1 codes (two per byte), or fp8 bytes.  Largest magnitude and
@@ -146,51 +175,92 @@ __global__ __launch_bounds__(256) void downcast_rows_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// downcast, source contiguous along r (quantised axis strided): a thread owns
-// NV adjacent columns and walks the 32 rows of one group, keeping them in registers.
+// downcast, source contiguous along r (quantised axis strided), any alignment: a thread owns one column and
+// walks the 32 rows of one group.  The aligned case has the tile kernel below.
 // ---------------------------------------------------------------------------
-template <int DT, int NV>
+template <int DT>
 __global__ __launch_bounds__(256) void downcast_cols_kernel(
     const void *__restrict__ src, int64_t nb, int64_t G, int64_t nr, int64_t ssb, int64_t ssl,
     uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
     int64_t csr, int mode) {
-  // a workgroup covers 8 consecutive groups of 32 column sets: the 8 lanes that share a column set write 8 x 16
-  // consecutive bytes of codes of each of its columns (one 128-byte line) and 8 consecutive scale bytes.  The
-  // grid is ceil(n_rv / 32) * ceil(G / 8) * nb workgroups (launch_downcast).
-  int64_t n_rv = (nr + NV - 1) / NV;
-  int64_t blocks_r = (n_rv + 31) / 32;
+  // a workgroup covers 8 consecutive groups of 32 columns: the 8 lanes that share a column write 8 x 16
+  // consecutive bytes of its codes (one 128-byte line) and 8 consecutive scale bytes.  The grid is
+  // ceil(nr / 32) * ceil(G / 8) * nb workgroups (launch_downcast).
+  int64_t blocks_r = (nr + 31) / 32;
   int64_t g_chunks = (G + 7) / 8;
   int64_t bid = blockIdx.x;
   int64_t br = bid % blocks_r;
   int64_t t = bid / blocks_r;
   int64_t g = (t % g_chunks) * 8 + threadIdx.x % 8;
   int64_t b = t / g_chunks;
-  int64_t rv = br * 32 + threadIdx.x / 8;
-  if (rv >= n_rv || g >= G || b >= nb) return;
-  int64_t r0 = rv * NV;
+  int64_t r0 = br * 32 + threadIdx.x / 8;
+  if (r0 >= nr || g >= G || b >= nb) return;
   constexpr int ES = DT == TAMD_F32 ? 4 : 2;
   const char *base = (const char *)src + (b * ssb + g * 32 * ssl + r0) * ES;
-  float mx[NV];
+  float mx = 0.f;
+  float v[32];
 #pragma unroll
-  for (int c = 0; c < NV; ++c) mx[c] = 0.f;
-  if constexpr (NV == 1) {
-    float v[32];
+  for (int l = 0; l < 32; ++l) {
+    v[l] = load_as_f32<DT>(base, l * ssl);
+    mx = __builtin_fmaxf(mx, __builtin_fabsf(v[l]));
+  }
+  uint32_t sbyte;
+  float qs = group_scale(mx, mode, sbyte);
+  uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (int l = 0; l < 32; ++l) {
-      v[l] = load_as_f32<DT>(base, l * ssl);
-      mx[0] = __builtin_fmaxf(mx[0], __builtin_fabsf(v[l]));
-    }
-    uint32_t sbyte;
-    float qs = group_scale(mx[0], mode, sbyte);
-    uint32_t w[4] = {0, 0, 0, 0};
-#pragma unroll
-    for (int l = 0; l < 32; l += 2) w[l >> 3] |= e2m1_pair(v[l] * qs, v[l + 1] * qs) << (4 * (l & 7));
-    *(uint4 *)(vals + b * vsb + r0 * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-    scales[b * csb + r0 * csr + g] = (uint8_t)sbyte;
-  } else {
+  for (int l = 0; l < 32; l += 2) w[l >> 3] |= e2m1_pair(v[l] * qs, v[l + 1] * qs) << (4 * (l & 7));
+  *(uint4 *)(vals + b * vsb + r0 * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+  scales[b * csb + r0 * csr + g] = (uint8_t)sbyte;
+}
+
+// ---------------------------------------------------------------------------
+// downcast, source contiguous along r, 16-byte aligned: a workgroup quantises a tile of GT groups x 32*NV
+// columns.  A load instruction of a wave reads 512 contiguous bytes of two source rows (a thread keeps the 32
+// rows of its NV columns in registers, as above); the codes pass through LDS so that they leave as GT x 16
+// contiguous bytes per column.  The source is read once and the codes are not read back here: both bypass the
+// caches' retention (non-temporal), which is worth a quarter of the time on this memory system.
+// ---------------------------------------------------------------------------
+// groups per tile: 64 KiB of codes in LDS either way
+template <int DT>
+constexpr int kTileGroups = DT == TAMD_F32 ? 32 : 16;
+template <int DT>
+constexpr int kTileCols = 32 * (DT == TAMD_F32 ? 4 : 8);
+template <int DT>
+constexpr size_t kTileLds = (size_t)kTileCols<DT> * kTileGroups<DT> * 17;
+
+template <int DT>
+__global__ __launch_bounds__(256) void downcast_cols_tile_kernel(
+    const void *__restrict__ src, int64_t nb, int64_t G, int64_t nr, int64_t ssb, int64_t ssl,
+    uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, uint8_t *__restrict__ scales, int64_t csb,
+    int64_t csr, int mode) {
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  constexpr int NV = 16 / ES;
+  constexpr int GT = kTileGroups<DT>;
+  constexpr int CW = kTileCols<DT>;
+  // s_codes[column][slot]: slot = group ^ (column / NV) % 8 keeps both the writes (two groups, 32 column sets
+  // per wave) and the reads (GT groups of 256 / GT columns per workgroup) spread over the banks
+  extern __shared__ uint4 s_tile[];
+  uint4 *s_codes = s_tile;
+  uint8_t *s_sc = (uint8_t *)(s_tile + CW * GT);
+  const int64_t tiles_r = (nr + CW - 1) / CW;
+  const int64_t g_chunks = (G + GT - 1) / GT;
+  const int64_t bid = blockIdx.x;
+  const int64_t br = bid % tiles_r;
+  const int64_t t = bid / tiles_r;
+  const int64_t gc = t % g_chunks;
+  const int64_t b = t / g_chunks;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int cs = lane % 32;  // the thread's column set
+  const int64_t col0 = br * CW + cs * NV;
+#pragma unroll 1
+  for (int pass = 0; pass < GT / 8; ++pass) {
+    const int gl = pass * 8 + wave * 2 + lane / 32;
+    const int64_t g = gc * GT + gl;
+    if (g >= G || col0 >= nr) continue;
+    const char *base = (const char *)src + (b * ssb + g * 32 * ssl + col0) * ES;
     uint4 raw[32];
 #pragma unroll
-    for (int l = 0; l < 32; ++l) raw[l] = *(const uint4 *)(base + (int64_t)l * ssl * ES);
+    for (int l = 0; l < 32; ++l) raw[l] = load_once(base + (int64_t)l * ssl * ES);
     auto elem = [&](int l, int c) -> float {
       const uint4 &q = raw[l];
       uint32_t w[4] = {q.x, q.y, q.z, q.w};
@@ -199,19 +269,51 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
       if constexpr (DT == TAMD_BF16) return bf16_bits_to_f32(h);
       return f16_bits_to_f32(h);
     };
+    float mx[NV];
+#pragma unroll
+    for (int c = 0; c < NV; ++c) mx[c] = 0.f;
 #pragma unroll
     for (int l = 0; l < 32; ++l)
 #pragma unroll
       for (int c = 0; c < NV; ++c) mx[c] = __builtin_fmaxf(mx[c], __builtin_fabsf(elem(l, c)));
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
+      bool has_nan = false;
+#pragma unroll
+      for (int l = 0; l < 32; l += 2) has_nan |= __builtin_isunordered(elem(l, c), elem(l + 1, c));
       uint32_t sbyte;
       float qs = group_scale(mx[c], mode, sbyte);
       uint32_t w[4] = {0, 0, 0, 0};
+      if (!has_nan && sbyte - 2u <= 251u) {
+        // the usual case: the instruction divides by the scale and packs, 1.5 operations per element
+        const float ds = bits_to_f32(sbyte << 23);
 #pragma unroll
-      for (int l = 0; l < 32; l += 2) w[l >> 3] |= e2m1_pair(elem(l, c) * qs, elem(l + 1, c) * qs) << (4 * (l & 7));
-      *(uint4 *)(vals + b * vsb + (r0 + c) * vsr + g * 16) = make_uint4(w[0], w[1], w[2], w[3]);
-      scales[b * csb + (r0 + c) * csr + g] = (uint8_t)sbyte;
+        for (int j = 0; j < 4; ++j) {
+          const float v[8] = {elem(8 * j, c),     elem(8 * j + 1, c), elem(8 * j + 2, c), elem(8 * j + 3, c),
+                              elem(8 * j + 4, c), elem(8 * j + 5, c), elem(8 * j + 6, c), elem(8 * j + 7, c)};
+          w[j] = e2m1_word_scaled(v, ds);
+        }
+      } else {
+#pragma unroll
+        for (int l = 0; l < 32; l += 2)
+          w[l >> 3] |= e2m1_pair(elem(l, c) * qs, elem(l + 1, c) * qs) << (4 * (l & 7));
+      }
+      const int cl = cs * NV + c;
+      s_codes[cl * GT + (gl ^ (cs & 7))] = make_uint4(w[0], w[1], w[2], w[3]);
+      s_sc[cl * GT + gl] = (uint8_t)sbyte;
+    }
+  }
+  __syncthreads();
+  const int64_t n_g = G - gc * GT < GT ? G - gc * GT : GT;
+  const int64_t n_c = nr - br * CW < CW ? nr - br * CW : CW;
+  uint8_t *vbase = vals + b * vsb + br * CW * vsr + gc * GT * 16;
+  uint8_t *sbase = scales + b * csb + br * CW * csr + gc * GT;
+  const int part = threadIdx.x % GT;
+  if (part < n_g) {
+#pragma unroll 4
+    for (int c = threadIdx.x / GT; c < n_c; c += 256 / GT) {
+      store_once(vbase + (int64_t)c * vsr + part * 16, s_codes[c * GT + (part ^ ((c / NV) & 7))]);
+      sbase[(int64_t)c * csr + part] = s_sc[c * GT + part];
     }
   }
 }
@@ -262,55 +364,178 @@ __global__ __launch_bounds__(256) void upcast_rows_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// upcast, destination contiguous along r: a thread owns NV columns of one group
+// upcast, destination contiguous along r, any alignment: a thread owns one column of one group.  The aligned
+// case has the tile kernel below.
 // ---------------------------------------------------------------------------
-template <int DT, int NV>
+template <int DT>
 __global__ __launch_bounds__(256) void upcast_cols_kernel(
     const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
     int64_t csb, int64_t csr, void *__restrict__ dst, int64_t nb, int64_t G, int64_t nr, int64_t dsb,
     int64_t dsl) {
-  // a workgroup covers 8 consecutive groups of 32 column sets: the 8 lanes that share a column set read 8 x 16
-  // consecutive bytes of each of its columns (one 128-byte line) and 8 consecutive scale bytes.  The grid is
-  // ceil(n_rv / 32) * ceil(G / 8) * nb workgroups (launch_upcast).
-  int64_t n_rv = (nr + NV - 1) / NV;
-  int64_t blocks_r = (n_rv + 31) / 32;
+  // a workgroup covers 8 consecutive groups of 32 columns: the 8 lanes that share a column read 8 x 16
+  // consecutive bytes of its codes (one 128-byte line) and 8 consecutive scale bytes.  The grid is
+  // ceil(nr / 32) * ceil(G / 8) * nb workgroups (launch_upcast).
+  int64_t blocks_r = (nr + 31) / 32;
   int64_t g_chunks = (G + 7) / 8;
   int64_t bid = blockIdx.x;
   int64_t br = bid % blocks_r;
   int64_t t = bid / blocks_r;
   int64_t g = (t % g_chunks) * 8 + threadIdx.x % 8;
   int64_t b = t / g_chunks;
-  int64_t rv = br * 32 + threadIdx.x / 8;
-  if (rv >= n_rv || g >= G || b >= nb) return;
-  int64_t r0 = rv * NV;
-  uint4 code[NV];
-  float mult[NV];
-  bool isn[NV];
-#pragma unroll
-  for (int c = 0; c < NV; ++c) {
-    code[c] = *(const uint4 *)(vals + b * vsb + (r0 + c) * vsr + g * 16);
-    uint32_t s = scales[b * csb + (r0 + c) * csr + g];
-    mult[c] = bits_to_f32(s << 23);
-    isn[c] = s == 0xFFu;
-  }
+  int64_t r0 = br * 32 + threadIdx.x / 8;
+  if (r0 >= nr || g >= G || b >= nb) return;
+  const uint4 code = *(const uint4 *)(vals + b * vsb + r0 * vsr + g * 16);
+  const uint32_t s = scales[b * csb + r0 * csr + g];
+  const float mult = bits_to_f32(s << 23);
+  const bool isn = s == 0xFFu;
   constexpr int ES = DT == TAMD_F32 ? 4 : 2;
   char *base = (char *)dst + (b * dsb + g * 32 * dsl + r0) * ES;
+  const uint32_t w[4] = {code.x, code.y, code.z, code.w};
 #pragma unroll
-  for (int l = 0; l < 32; ++l) {
-    float o[NV];
+  for (int l = 0; l < 32; ++l)
+    store_from_f32<DT>(base + (int64_t)l * dsl * ES, 0, dequant_one<DT>((w[l >> 3] >> (4 * (l & 7))) & 0xFu, mult, isn));
+}
+
+// Scale bytes for which 0.5 * 2^(s-127) and 6 * 2^(s-127) are normal numbers of the destination type: there the
+// product needs neither the clamp to the largest finite value nor any care about denormals.
+template <int DT>
+constexpr uint32_t kFastLo = DT == TAMD_F16 ? 127u - 13u : 3u;
+template <int DT>
+constexpr uint32_t kFastHi = DT == TAMD_F16 ? 127u + 13u : 252u;
+
+// Rows l and l+1 (the code pairs in byte BS of w[c]) of a thread's 16 / sizeof(element) columns, dequantised by the
+// conversion instruction and stored as two 16-byte pieces `pitch` bytes apart.
+template <int DT, int BS>
+TAMD_DEVICE void upcast_rows2_regs(const uint32_t *w, const float *mult, uint4 &r0, uint4 &r1) {
+  if constexpr (DT == TAMD_F32) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) v[c] = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[c], mult[c], BS);
+    r0 = make_uint4(f32_to_bits(v[0].x), f32_to_bits(v[1].x), f32_to_bits(v[2].x), f32_to_bits(v[3].x));
+    r1 = make_uint4(f32_to_bits(v[0].y), f32_to_bits(v[1].y), f32_to_bits(v[2].y), f32_to_bits(v[3].y));
+  } else {
+    uint32_t u[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      if constexpr (DT == TAMD_BF16) {
+        typedef __bf16 bf16x2v_t __attribute__((ext_vector_type(2)));
+        bf16x2v_t t = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[c], mult[c], BS);
+        u[c] = __builtin_bit_cast(uint32_t, t);
+      } else {
+        typedef _Float16 f16x2v_t __attribute__((ext_vector_type(2)));
+        f16x2v_t t = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[c], mult[c], BS);
+        u[c] = __builtin_bit_cast(uint32_t, t);
+      }
+    }
+    // u[c] = (row l, row l+1) of column c; a stored word is (column 2i, column 2i+1) of one row
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[i] = __builtin_amdgcn_perm(u[2 * i + 1], u[2 * i], 0x05040100u);
+      hi[i] = __builtin_amdgcn_perm(u[2 * i + 1], u[2 * i], 0x07060302u);
+    }
+    r0 = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    r1 = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+  }
+}
+template <int DT, int BS>
+TAMD_DEVICE void upcast_rows2(const uint32_t *w, const float *mult, char *p, int64_t pitch) {
+  uint4 r0, r1;
+  upcast_rows2_regs<DT, BS>(w, mult, r0, r1);
+  store_once(p, r0);
+  store_once(p + pitch, r1);
+}
+
+// ---------------------------------------------------------------------------
+// upcast, destination contiguous along r, 16-byte aligned: the mirror image of downcast_cols_tile_kernel.  The
+// codes and scales of a tile of GT groups x 32*NV columns come in as GT x 16 contiguous bytes per column, pass
+// through LDS, and a store instruction of a wave writes 512 contiguous bytes of two destination rows.
+// ---------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void upcast_cols_tile_kernel(
+    const uint8_t *__restrict__ vals, int64_t vsb, int64_t vsr, const uint8_t *__restrict__ scales,
+    int64_t csb, int64_t csr, void *__restrict__ dst, int64_t nb, int64_t G, int64_t nr, int64_t dsb,
+    int64_t dsl) {
+  constexpr int ES = DT == TAMD_F32 ? 4 : 2;
+  constexpr int NV = 16 / ES;
+  constexpr int GT = kTileGroups<DT>;
+  constexpr int CW = kTileCols<DT>;
+  extern __shared__ uint4 s_tile[];
+  uint4 *s_codes = s_tile;
+  uint8_t *s_sc = (uint8_t *)(s_tile + CW * GT);
+  const int64_t tiles_r = (nr + CW - 1) / CW;
+  const int64_t g_chunks = (G + GT - 1) / GT;
+  const int64_t bid = blockIdx.x;
+  const int64_t br = bid % tiles_r;
+  const int64_t t = bid / tiles_r;
+  const int64_t gc = t % g_chunks;
+  const int64_t b = t / g_chunks;
+  const int64_t n_g = G - gc * GT < GT ? G - gc * GT : GT;
+  const int64_t n_c = nr - br * CW < CW ? nr - br * CW : CW;
+  const uint8_t *vbase = vals + b * vsb + br * CW * vsr + gc * GT * 16;
+  const uint8_t *sbase = scales + b * csb + br * CW * csr + gc * GT;
+  const int part = threadIdx.x % GT;
+  if (part < n_g) {
+#pragma unroll 4
+    for (int c = threadIdx.x / GT; c < n_c; c += 256 / GT) {
+      s_codes[c * GT + (part ^ ((c / NV) & 7))] = load_once(vbase + (int64_t)c * vsr + part * 16);
+      s_sc[c * GT + part] = sbase[(int64_t)c * csr + part];
+    }
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int cs = lane % 32;
+  const int64_t col0 = br * CW + cs * NV;
+#pragma unroll 1
+  for (int pass = 0; pass < GT / 8; ++pass) {
+    const int gl = pass * 8 + wave * 2 + lane / 32;
+    const int64_t g = gc * GT + gl;
+    if (g >= G || col0 >= nr) continue;
+    uint4 code[NV];
+    float mult[NV];
+    bool isn[NV];
+    bool fast = true;
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
-      uint32_t w[4] = {code[c].x, code[c].y, code[c].z, code[c].w};
-      o[c] = dequant_one<DT>((w[l >> 3] >> (4 * (l & 7))) & 0xFu, mult[c], isn[c]);
+      const int cl = cs * NV + c;
+      code[c] = s_codes[cl * GT + (gl ^ (cs & 7))];
+      uint32_t s = s_sc[cl * GT + gl];
+      mult[c] = bits_to_f32(s << 23);
+      isn[c] = s == 0xFFu;
+      fast &= s - kFastLo<DT> <= kFastHi<DT> - kFastLo<DT>;
     }
-    char *p = base + (int64_t)l * dsl * ES;
-    if constexpr (NV == 1) {
-      store_from_f32<DT>(p, 0, o[0]);
-    } else if constexpr (DT == TAMD_F32) {
-      *(float4 *)p = make_float4(o[0], o[1], o[2], o[3]);
-    } else {
-      *(uint4 *)p = make_uint4(pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3]), pack2<DT>(o[4], o[5]),
-                               pack2<DT>(o[6], o[7]));
+    char *base = (char *)dst + (b * dsb + g * 32 * dsl + col0) * ES;
+    if (fast) {
+      // the usual case: every product code * scale is a normal number of the destination type, and the
+      // conversion instruction yields it for two rows of a column at once
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t w[NV];
+#pragma unroll
+        for (int c = 0; c < NV; ++c) w[c] = j == 0 ? code[c].x : (j == 1 ? code[c].y : (j == 2 ? code[c].z : code[c].w));
+        upcast_rows2<DT, 0>(w, mult, base + (int64_t)(8 * j + 0) * dsl * ES, dsl * ES);
+        upcast_rows2<DT, 1>(w, mult, base + (int64_t)(8 * j + 2) * dsl * ES, dsl * ES);
+        upcast_rows2<DT, 2>(w, mult, base + (int64_t)(8 * j + 4) * dsl * ES, dsl * ES);
+        upcast_rows2<DT, 3>(w, mult, base + (int64_t)(8 * j + 6) * dsl * ES, dsl * ES);
+      }
+      continue;
+    }
+#pragma unroll
+    for (int l = 0; l < 32; ++l) {
+      float o[NV];
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        uint32_t w[4] = {code[c].x, code[c].y, code[c].z, code[c].w};
+        o[c] = dequant_one<DT>((w[l >> 3] >> (4 * (l & 7))) & 0xFu, mult[c], isn[c]);
+      }
+      char *p = base + (int64_t)l * dsl * ES;
+      if constexpr (DT == TAMD_F32) {
+        store_once(p, make_uint4(f32_to_bits(o[0]), f32_to_bits(o[1]), f32_to_bits(o[2]), f32_to_bits(o[3])));
+      } else {
+        store_once(p, make_uint4(pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3]), pack2<DT>(o[4], o[5]),
+                                 pack2<DT>(o[6], o[7])));
+      }
     }
   }
 }
@@ -339,14 +564,16 @@ int launch_downcast(const void *src, int64_t nb, int64_t L, int64_t nr, int64_t 
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(src, 16) && (ssb * ES) % 16 == 0 && (ssl * ES) % 16 == 0;
   if (vec) {
-    int64_t blocks = ((nr / NV + 31) / 32) * ((G + 7) / 8) * nb;
+    constexpr int CW = kTileCols<DT>, GT = kTileGroups<DT>;
+    int64_t blocks = ((nr + CW - 1) / CW) * ((G + GT - 1) / GT) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-    downcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
-                                                                        scales, csb, csr, mode);
+    if (int rc = raise_lds_limit_once((const void *)downcast_cols_tile_kernel<DT>)) return rc;
+    downcast_cols_tile_kernel<DT><<<dim3((unsigned)blocks), 256, kTileLds<DT>, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
+                                                                         scales, csb, csr, mode);
   } else {
     int64_t blocks = ((nr + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-    downcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
+    downcast_cols_kernel<DT><<<dim3((unsigned)blocks), 256, 0, st>>>(src, nb, G, nr, ssb, ssl, vals, vsb, vsr,
                                                                        scales, csb, csr, mode);
   }
   return launch_status();
@@ -372,14 +599,16 @@ int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *
   constexpr int NV = 16 / ES;
   bool vec = nr % NV == 0 && aligned(dst, 16) && (dsb * ES) % 16 == 0 && (dsl * ES) % 16 == 0;
   if (vec) {
-    int64_t blocks = ((nr / NV + 31) / 32) * ((G + 7) / 8) * nb;
+    constexpr int CW = kTileCols<DT>, GT = kTileGroups<DT>;
+    int64_t blocks = ((nr + CW - 1) / CW) * ((G + GT - 1) / GT) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-    upcast_cols_kernel<DT, NV><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
-                                                                      nr, dsb, dsl);
+    if (int rc = raise_lds_limit_once((const void *)upcast_cols_tile_kernel<DT>)) return rc;
+    upcast_cols_tile_kernel<DT><<<dim3((unsigned)blocks), 256, kTileLds<DT>, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
+                                                                       nr, dsb, dsl);
   } else {
     int64_t blocks = ((nr + 31) / 32) * ((G + 7) / 8) * nb;
     if (blocks > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-    upcast_cols_kernel<DT, 1><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
+    upcast_cols_kernel<DT><<<dim3((unsigned)blocks), 256, 0, st>>>(vals, vsb, vsr, scales, csb, csr, dst, nb, G,
                                                                      nr, dsb, dsl);
   }
   return launch_status();
