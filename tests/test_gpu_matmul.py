@@ -448,6 +448,25 @@ def test_dense_16bit_weights(M, K, N, dtype, k_contiguous, device):
     check(out, ref)
 
 
+@pytest.mark.parametrize("M,K,N", [(2048, 5760, 128), (100, 136, 40), (17, 8, 100), (5, 2888, 128), (64, 64, 8), (333, 4096, 72)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_narrow_dense_product(M, K, N, dtype, out_f32, device):
+    """N <= 128 goes to the kernel without LDS staging (16 rows x 64 columns per workgroup, K split over the waves):
+    ragged edges in M, N and K, bias on and off, float32 output, both storage orders of the weights.
+    (2048, 5760, 128) is the gate matmul of the reference's bench_mlp."""
+    torch.manual_seed(M + N)
+    x = torch.randn(M, K).to(dtype)
+    w = (torch.randn(K, N) * 0.05).to(dtype)
+    bias = torch.randn(N) if N != 40 else None
+    pc = PrecisionConfig(out_dtype=torch.float32) if out_f32 else None
+    for wd in (w.to(device), w.to(device).T.contiguous().T):
+        out = matmul(x.to(device), wd, None if bias is None else bias.to(device), precision_config=pc)
+        ref = MR.matmul_ref(x, w, bias)
+        assert out.dtype == (torch.float32 if out_f32 else dtype) and tuple(out.shape) == (M, N)
+        check(out, ref if not out_f32 else (x.float() @ w.float() + (0 if bias is None else bias)))
+
+
 @pytest.mark.parametrize("block_m", [None, 16, 64])
 @pytest.mark.parametrize("act", [False, True])
 def test_ragged_16bit_weights(block_m, act, device):

@@ -1,6 +1,7 @@
 // Bandwidth kernels next to the matmul: the top-k combine (sum over the middle
 // axis with optional mask / scale) and the standalone interleaved SwiGLU.
 #include "common.h"
+#include <type_traits>
 
 namespace tamd {
 
@@ -240,8 +241,8 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
 #pragma unroll
     for (int j = 0; j < PV; ++j) acc[j] = 0.f;
     if (c0 < S1) {
-      for (int64_t r = 0; r < a.R; ++r) {
-        float v[PV];
+      // PV values of row r of the reduced axis
+      auto load_row = [&](int64_t r, float (&v)[PV]) {
         const int64_t xo = s0 * a.xs0 + r * a.xsr;
         if (PV == 8 && vec_in) {  // unit inner stride, 8 columns inside S1, 8-element alignment of every row
           if (xsz == 4) {
@@ -267,6 +268,59 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
 #pragma unroll
           for (int j = 0; j < PV; ++j) v[j] = c0 + j < S1 ? load_elem_f32(a.x, a.x_dtype, xo + (c0 + j) * a.xs1) : 0.f;
         }
+      };
+      int64_t r = 0;
+      if (PV == 8 && vec_in && !a.x_mx_scale && !a.scale && !a.mask) {
+        // plain sums (the top-k combine): four rows are fetched together -- raw loads first, conversions after, with
+        // the element size fixed outside so that no branch separates the loads -- and added in the order r = 0, 1, ...
+        auto batches = [&](auto xs_tag) {
+          constexpr int XS = decltype(xs_tag)::value;
+          constexpr int NQ = XS == 4 ? 2 : 1;
+          for (; r + 4 <= a.R; r += 4) {
+            uint4 q[4][NQ];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const uint8_t *src = (const uint8_t *)a.x + (s0 * a.xs0 + (r + u) * a.xsr + c0) * XS;
+              if constexpr (XS == 1) {
+                const uint2 h = *(const uint2 *)src;
+                q[u][0] = make_uint4(h.x, h.y, 0, 0);
+              } else {
+#pragma unroll
+                for (int n = 0; n < NQ; ++n) q[u][n] = *(const uint4 *)(src + 16 * n);
+              }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              float v[8];
+              if constexpr (XS == 4) {
+                v[0] = bits_to_f32(q[u][0].x), v[1] = bits_to_f32(q[u][0].y), v[2] = bits_to_f32(q[u][0].z), v[3] = bits_to_f32(q[u][0].w);
+                v[4] = bits_to_f32(q[u][NQ - 1].x), v[5] = bits_to_f32(q[u][NQ - 1].y), v[6] = bits_to_f32(q[u][NQ - 1].z), v[7] = bits_to_f32(q[u][NQ - 1].w);
+              } else if constexpr (XS == 2) {
+                const uint32_t w[4] = {q[u][0].x, q[u][0].y, q[u][0].z, q[u][0].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  v[2 * j] = a.x_dtype == TAMD_BF16 ? bf16_bits_to_f32(w[j] & 0xFFFFu) : f16_bits_to_f32(w[j] & 0xFFFFu);
+                  v[2 * j + 1] = a.x_dtype == TAMD_BF16 ? bf16_bits_to_f32(w[j] >> 16) : f16_bits_to_f32(w[j] >> 16);
+                }
+              } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                  const int b = (int)(((j < 4 ? q[u][0].x : q[u][0].y) >> (8 * (j & 3))) & 0xFFu);
+                  v[j] = a.x_dtype == TAMD_FP8_E4M3 ? __builtin_amdgcn_cvt_f32_fp8(b, 0) : __builtin_amdgcn_cvt_f32_bf8(b, 0);
+                }
+              }
+#pragma unroll
+              for (int j = 0; j < PV; ++j) acc[j] += v[j % 8] * flex_in;
+            }
+          }
+        };
+        if (xsz == 1) batches(std::integral_constant<int, 1>{});
+        else if (xsz == 2) batches(std::integral_constant<int, 2>{});
+        else batches(std::integral_constant<int, 4>{});
+      }
+      for (; r < a.R; ++r) {
+        float v[PV];
+        load_row(r, v);
 #pragma unroll
         for (int j = 0; j < PV; ++j) {
           const int64_t c = c0 + j;

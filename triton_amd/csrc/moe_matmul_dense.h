@@ -182,10 +182,172 @@ int launch_w16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   return launch_status();
 }
 
+// ---------------------------------------------------------------------------
+// Narrow outputs (N <= 128: the gate matmul, tokens x d_model times d_model x n_experts): one dense product whose
+// weights are small and whose activations are read once.  The tiled kernel above would give such a problem a
+// handful of half-empty 256-column tiles with a long, latency-bound K loop each.  Here a workgroup owns 16 rows x
+// 64 columns and its four waves split K: wave w takes the 64-K blocks w, w + 4, ...  Both operands are
+// K-contiguous; a block is 16 + 64 lines of 128 bytes, copied by DMA whole lines at a time (8 lanes per line)
+// into a ring of three stages that belongs to the wave alone -- so the loop has no barrier: a wave waits for its
+// own copies, reads v_mfma_f32_16x16x32 operands (lane (c = lane % 16, g = lane / 16): K values 8g .. 8g+7 of
+// row / column c; 16-byte chunks swizzled by the line index) and requests the block two ahead.  The four partial
+// sums meet in LDS; bias, scales and the cast follow.
+// ---------------------------------------------------------------------------
+typedef float f32x4s_t __attribute__((ext_vector_type(4)));
+template <int XDT>
+TAMD_DEVICE f32x4s_t mma16x16x32(uint4 a, uint4 b, f32x4s_t c) {
+  if constexpr (XDT == TAMD_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+
+constexpr int SKINNY_COLS = 64;                     // columns of a workgroup
+constexpr int SKINNY_PITCH = 68;                    // floats per row of a partial sum in LDS (padded)
+constexpr int SKINNY_STAGE = (16 + 64) * 128;       // bytes of one 64-K block: 16 rows, then 64 columns
+constexpr int SKINNY_RING = 3;
+constexpr int SKINNY_LDS = 4 * SKINNY_RING * SKINNY_STAGE + 4 * 16 * SKINNY_PITCH * 4;
+
+template <int XDT>
+__global__ __launch_bounds__(256) void mm_skinny16_kernel(tamd_matmul_args a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr uint32_t kOob = 0x7FFFFFFFu;
+  float *red = (float *)(lds + 4 * SKINNY_RING * SKINNY_STAGE);
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+  const int c = lane % 16, g = lane / 16;
+  const int M = a.M, N = a.N, K = a.K;
+  const int row0 = blockIdx.x * 16, col0 = blockIdx.y * SKINNY_COLS;
+  const v4i_t rx = make_rsrc(a.x, kOob), rw = make_rsrc(a.w, kOob);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const uint32_t ring = lds_base + wave * SKINNY_RING * SKINNY_STAGE;
+  const uint8_t *ringp = lds + wave * SKINNY_RING * SKINNY_STAGE;
+  // copy instruction i moves lines 8i .. 8i+7 of a stage: lane -> (line 8i + lane / 8, 16-byte slot lane % 8), the
+  // slot holding chunk slot ^ (line % 8) of the line.  Rows past M and columns past N repeat the last one (their
+  // results are not stored); chunks past K are not read (zeros).
+  const int slot = lane % 8;
+  uint32_t src_off[10];
+  int src_chunk[10];
+#pragma unroll
+  for (int i = 0; i < 10; ++i) {
+    const int line = (i < 2 ? i : i - 2) * 8 + lane / 8;
+    src_chunk[i] = slot ^ (line & 7);
+    if (i < 2) {
+      const int row = row0 + line < M ? row0 + line : M - 1;
+      src_off[i] = (uint32_t)((int64_t)row * a.x_stride_m * 2) + src_chunk[i] * 16;
+    } else {
+      const int col = col0 + line < N ? col0 + line : N - 1;
+      src_off[i] = (uint32_t)((int64_t)col * a.w_stride_n * 2) + src_chunk[i] * 16;
+    }
+  }
+  const int n_blocks = (K + 63) / 64;
+  auto issue = [&](int kb, int st) {  // block kb (may lie past the end: nothing is read) into stage st
+    const uint32_t dst = ring + st * SKINNY_STAGE;
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+      const uint32_t kill = kb * 64 + src_chunk[i] * 8 < K ? 0u : kOob;
+      dma16(i < 2 ? rx : rw, dst + i * 1024, src_off[i] | kill, (uint32_t)kb * 128u);
+    }
+  };
+  f32x4s_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = f32x4s_t{0.f, 0.f, 0.f, 0.f};
+  issue(wave, 0);
+  issue(wave + 4, 1);
+  int st = 0;
+#pragma unroll 1
+  for (int kb = wave; kb < n_blocks; kb += 4) {
+    wait_vmcnt<10>();  // copies complete in order: all but the newest block's ten have landed
+    const uint8_t *sp = ringp + st * SKINNY_STAGE;
+    uint4 av[2], bv[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      av[t] = *(const uint4 *)(sp + c * 128 + (((t * 4 + g) ^ (c & 7)) * 16));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int line = j * 16 + c;
+        bv[t][j] = *(const uint4 *)(sp + 2048 + line * 128 + (((t * 4 + g) ^ (line & 7)) * 16));
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // operands are in registers: the stage two ahead may reuse ...
+    const int nst = st == 0 ? 2 : st - 1;                // ... the stage read one iteration ago
+    issue(kb + 8, nst);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = mma16x16x32<XDT>(av[t], bv[t][j], acc[j]);
+    st = st == 2 ? 0 : st + 1;
+  }
+  wait_dma();
+  // element i of fragment j is row 4g + i, column 16j + c
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[(wave * 16 + g * 4 + i) * SKINNY_PITCH + j * 16 + c] = acc[j][i];
+  __syncthreads();
+  // thread -> row tid / 16, four columns
+  const int r = tid / 16, cq = (tid % 16) * 4;
+  if (row0 + r >= M) return;
+  float flex = 1.0f;
+  if (a.x_scale) flex *= *a.x_scale;
+  if (a.w_scale) flex *= *a.w_scale;
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int idx = r * SKINNY_PITCH + cq + e;
+    const float v = (red[idx] + red[16 * SKINNY_PITCH + idx]) + (red[32 * SKINNY_PITCH + idx] + red[48 * SKINNY_PITCH + idx]);
+    const int col = col0 + cq + e;
+    const float b = (a.bias && col < N) ? load_any_f32(a.bias, a.bias_dtype, col) : 0.f;
+    o[e] = (v * flex + b) * a.out_alpha;
+  }
+  const int64_t base = (int64_t)(row0 + r) * a.y_stride_m + col0 + cq;
+  if (a.y_dtype == TAMD_F32) {
+    float *yp = (float *)a.y + base;
+    if (col0 + cq + 4 <= N && ((uintptr_t)yp & 15) == 0) *(float4 *)yp = make_float4(o[0], o[1], o[2], o[3]);
+    else
+      for (int e = 0; e < 4 && col0 + cq + e < N; ++e) yp[e] = o[e];
+  } else {
+    uint16_t *yp = (uint16_t *)a.y + base;
+    uint32_t h[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = a.y_dtype == TAMD_BF16 ? f32_to_bf16_bits(o[e]) : f32_to_f16_bits(o[e]);
+    if (col0 + cq + 4 <= N && ((uintptr_t)yp & 7) == 0) *(uint2 *)yp = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+    else
+      for (int e = 0; e < 4 && col0 + cq + e < N; ++e) yp[e] = (uint16_t)h[e];
+  }
+}
+
+// Whether the narrow kernel covers the problem: one dense product (no ragged / batched / gathered rows, no per-row
+// factors, no activation, no flexpoint or microscaled output), K-contiguous weights, N <= 128, both operands
+// addressable with 32-bit byte offsets.
+inline bool skinny16_applicable(const tamd_matmul_args &a) {
+  if (a.N > 128 || a.N < 1 || a.M < 1 || a.n_experts != 1 || a.w_stride_k != 1 || a.K % 8 != 0) return false;
+  if (a.block_schedule || a.slice_sizes || a.gather_indx || a.scatter_indx || a.betas || a.gammas) return false;
+  if (a.activation != TAMD_ACT_NONE || a.y_expected_scale || a.y_actual_scale || a.y_mx_scale || a.x_mx_scale) return false;
+  if (a.y_dtype != a.x_dtype && a.y_dtype != TAMD_F32) return false;
+  if (a.force_variant != 0) return false;
+  if (!aligned(a.w, 16) || (a.w_stride_n * 2) % 16 != 0 || !aligned(a.x, 16) || (a.x_stride_m * 2) % 16 != 0) return false;
+  if (a.x_stride_m < 0 || a.w_stride_n < 0) return false;
+  const int64_t lim = 0x7FFFFF00;
+  if (((int64_t)a.M * a.x_stride_m + a.K) * 2 >= lim || ((int64_t)a.N * a.w_stride_n + a.K) * 2 >= lim) return false;
+  return true;
+}
+
+template <int XDT>
+int launch_skinny16(const tamd_matmul_args &a, hipStream_t st) {
+  const int64_t gm = ((int64_t)a.M + 15) / 16;
+  if (gm > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
+  auto kern = mm_skinny16_kernel<XDT>;
+  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
+  kern<<<dim3((unsigned)gm, (unsigned)((a.N + SKINNY_COLS - 1) / SKINNY_COLS)), 256, SKINNY_LDS, st>>>(a);
+  return launch_status();
+}
+
 // 16-bit activations x 16-bit weights of the same type.  Returns TAMD_E_UNSUPPORTED / _ALIGNMENT for layouts
 // the kernel does not cover.
 template <int XDT>
 int dispatch_w16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
+  if (skinny16_applicable(a)) return launch_skinny16<XDT>(a, st);
   dense_grid(a, block_m, grid_m);
   const bool kc = a.w_stride_k == 1, nc = a.w_stride_n == 1;
   if (!kc && !nc) return TAMD_E_UNSUPPORTED;

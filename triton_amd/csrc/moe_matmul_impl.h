@@ -280,13 +280,29 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
   // per-row factors: lane L fetches those of row L % 32 of every fragment up front (one round trip to memory);
   // an element then takes its row's pair from that lane
   float beta_of[NFR], gamma_of[NFR];
+  const bool has_beta = ROWSC && a.betas != nullptr, has_gamma = ROWSC && a.gammas != nullptr;
   if constexpr (ROWSC) {
 #pragma unroll
     for (int i = 0; i < NFR; ++i) {
       const int r = i * 32 + c32;
       const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);  // expert-sorted row
-      beta_of[i] = a.betas ? a.betas[erow] : 1.0f;
-      gamma_of[i] = a.gammas ? a.gammas[erow] : 1.0f;
+      beta_of[i] = has_beta ? a.betas[erow] : 1.0f;
+      gamma_of[i] = has_gamma ? a.gammas[erow] : 1.0f;
+    }
+  }
+  // destination rows of the 16-byte chunks this thread copies out at the end (chunk id = tid + 256 u): fetched
+  // now, so that the scatter indices arrive while the values are computed
+  constexpr bool PRE = YDT >= 0 && YDT != TAMD_F32;
+  constexpr int OSZ_C = YDT == TAMD_FP8_E4M3 || YDT == TAMD_FP8_E5M2 ? 1 : 2;
+  constexpr int CPR_C = OUT_COLS * OSZ_C / 16;          // chunks per tile row
+  constexpr int MAXU = PRE ? NFR * 32 * CPR_C / 256 : 1;  // chunks per thread
+  int dst_row[MAXU];
+  if constexpr (PRE) {
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      const int r = (tid + u * 256) / CPR_C;
+      const int erow = t.start_m + t.off_m + (r < t.rows ? r : t.rows - 1);
+      dst_row[u] = a.scatter_indx ? a.scatter_indx[erow] : erow;
     }
   }
   __syncthreads();
@@ -298,9 +314,19 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
       float v[NF];
       float gamma = 1.0f;
       if constexpr (ROWSC) {
-        const int src_lane = (j >> 2) * 8 + h * 4 + (j & 3);
-        const float beta = __shfl(beta_of[i], src_lane);
-        gamma = __shfl(gamma_of[i], src_lane);
+        // the factors of row 32 i + l sit in lane l: lanes of half h need l = 8 (j / 4) + 4 h + j % 4
+        const int l0 = (j >> 2) * 8 + (j & 3);
+        float beta = 1.0f;
+        if (has_beta) {
+          const float b0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0));
+          const float b1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0 + 4));
+          beta = h ? b1 : b0;
+        }
+        if (has_gamma) {
+          const float g0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0));
+          const float g1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0 + 4));
+          gamma = h ? g1 : g0;
+        }
 #pragma unroll
         for (int f = 0; f < NF; ++f) v[f] = __builtin_fmaf(acc[i][f][j], flex, bias_a[f] * beta);
       } else {
@@ -405,6 +431,27 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
     const int epc = 16 / osz;                 // outputs per 16-byte chunk
     const int cpr = OUT_COLS / epc;           // chunks per tile row
     const int n_chunks = t.rows * cpr;
+    if constexpr (PRE) {
+#pragma unroll
+      for (int u = 0; u < MAXU; ++u) {
+        const int id = tid + u * 256;
+        if (id >= n_chunks) break;
+        const int r = id / CPR_C, c = (id - r * CPR_C) * (16 / OSZ_C);
+        const int64_t dst = dst_row[u];
+        if (dst < 0) continue;
+        const int gcol = tile_out0 + c;
+        if (gcol >= n_out) continue;
+        uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + dst * a.y_stride_m + gcol) * OSZ_C;
+        const uint8_t *sp = ob + (r * OUT_COLS + c) * OSZ_C;
+        if (gcol + 16 / OSZ_C <= n_out && ((uintptr_t)yp & 15) == 0) {
+          *(uint4 *)yp = *(const uint4 *)sp;
+        } else {
+          const int n_b = (n_out - gcol < 16 / OSZ_C ? n_out - gcol : 16 / OSZ_C) * OSZ_C;
+          for (int e = 0; e < n_b; ++e) yp[e] = sp[e];
+        }
+      }
+      return;
+    }
     // eight chunks per thread at a time, so that the scatter indices of a batch are fetched together
     for (int id0 = tid; id0 < n_chunks; id0 += 256 * 8) {
       int64_t dsts[8];
@@ -653,35 +700,46 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       }
   };
 
+  // fp8 path: A fragments of the two 64-K halves of a stage and the activations' scale operands
+  i32x8_t af8[FP8 ? 2 : 1][FP8 ? NFR : 1];
+  int sa8[FP8 ? NFR : 1];
+  auto fp8_read_frags = [&](const uint8_t *buf, int s, i32x8_t *af) {
+    const int swz = (c32 >> 1) & 7;
+#pragma unroll
+    for (int i = 0; i < NFR; ++i) {
+      const uint8_t *row = buf + (i * 32 + c32) * A_ROW_BYTES;
+      const uint4 lo = *(const uint4 *)(row + (((4 * s + h) ^ swz) * 16));
+      const uint4 hi = *(const uint4 *)(row + (((4 * s + 2 + h) ^ swz) * 16));
+      af[i] = i32x8_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    }
+  };
+  // first-half fragments and scale operands of stage `it`: issued together with the weight reads of the stage, so
+  // that their latency passes while the next stage's copies are requested
+  auto fp8_read0 = [&](int it) {
+    if constexpr (FP8) {
+      if (!wave_live) return;
+      const uint8_t *buf = lds + (it & 1) * A_STAGE;
+      fp8_read_frags(buf, 0, af8[0]);
+      // A scale operand: lane half h supplies K block h of an MFMA; byte 0 is the group of s = 0, byte 2 of s = 1
+#pragma unroll
+      for (int i = 0; i < NFR; ++i)
+        sa8[i] = x_mx ? (int)(as_buf[((it & 1) * 4 + h) * AS_ROWS + i * 32 + c32] |
+                              (as_buf[((it & 1) * 4 + 2 + h) * AS_ROWS + i * 32 + c32] << 16))
+                      : 0x7F7F7F7F;
+    }
+  };
+
   auto compute = [&](int it, auto qc) {
     constexpr int q = decltype(qc)::value;
     if (!wave_live) return;
     const uint8_t *buf = lds + (it & 1) * A_STAGE;
     if constexpr (FP8) {
-      // one stage = 128 K = two scaled MFMAs per (row fragment, column fragment)
+      // one stage = 128 K = two scaled MFMAs per (row fragment, column fragment); the fragments of the first half
+      // and the activations' scale operands are already in registers (fp8_read0)
       constexpr int CBSZ = XDT == TAMD_FP8_E5M2 ? 1 : 0;
-      auto read_frags = [&](int s, i32x8_t *af) {
-        const int swz = (c32 >> 1) & 7;
-#pragma unroll
-        for (int i = 0; i < NFR; ++i) {
-          const uint8_t *row = buf + (i * 32 + c32) * A_ROW_BYTES;
-          const uint4 lo = *(const uint4 *)(row + (((4 * s + h) ^ swz) * 16));
-          const uint4 hi = *(const uint4 *)(row + (((4 * s + 2 + h) ^ swz) * 16));
-          af[i] = i32x8_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
-      };
-      i32x8_t af[2][NFR];
-      read_frags(0, af[0]);
-      // A scale operand: lane half h supplies K block h of an MFMA; byte 0 is the group of s = 0, byte 2 of s = 1
-      int sa[NFR];
-#pragma unroll
-      for (int i = 0; i < NFR; ++i)
-        sa[i] = x_mx ? (int)(as_buf[((it & 1) * 4 + h) * AS_ROWS + i * 32 + c32] |
-                             (as_buf[((it & 1) * 4 + 2 + h) * AS_ROWS + i * 32 + c32] << 16))
-                     : 0x7F7F7F7F;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        if (s == 0) read_frags(1, af[1]);
+        if (s == 0) fp8_read_frags(buf, 1, af8[1]);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           const uint4 r = raw[f][s];
@@ -689,10 +747,10 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
           for (int i = 0; i < NFR; ++i) {
             if (s == 0)
-              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[0][i], bf, acc[i][f], CBSZ, 4, 0, sa[i], 0,
+              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[0][i], bf, acc[i][f], CBSZ, 4, 0, sa8[i], 0,
                                                                         (int)scw[f]);
             else
-              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[1][i], bf, acc[i][f], CBSZ, 4, 2, sa[i], 1,
+              acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[1][i], bf, acc[i][f], CBSZ, 4, 2, sa8[i], 1,
                                                                         (int)scw[f]);
           }
         }
@@ -728,6 +786,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       wait_dma();
       __syncthreads();
       load_b(it);
+      fp8_read0(it);
       issue_a(it + 1);
       issue_as(it + 1);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled

@@ -196,6 +196,11 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         # unquantised weights with unit stride along N whose rows do not start on 16-byte boundaries: the kernel copies
         # 16 bytes at a time, so they are laid out with unit stride along K instead (same values)
         w = w.transpose(-1, -2).contiguous().transpose(-1, -2)
+    if not b_fp4 and w.ndim == 2 and w.shape[-1] <= 128 and w.stride(-2) != 1 and w.shape[-2] % 8 == 0 \
+            and a_ragged_metadata is None and gather_indx is None and scatter_indx is None:
+        # a narrow dense product (the gate matmul: hidden -> expert logits): the kernel for it reads both operands
+        # along K, so weights stored with unit stride along N are turned once (a few hundred KB)
+        w = w.transpose(-1, -2).contiguous().transpose(-1, -2)
     _lib.require_gpu(a, "a")
     _lib.require_gpu(w, "b")
     assert a.stride(-1) == 1 or a.shape[-1] == 1, "a must be contiguous along K"
