@@ -226,6 +226,27 @@ TAMD_DEVICE v4i_t make_rsrc(const void *base, uint32_t num_records) {
 
 constexpr int A_ROW_BYTES = 128;       // LDS bytes per activation row per stage (64 K of 16-bit, 128 K of fp8)
 constexpr int B_BYTES = 4 * 64 * 64;   // 4 waves x 64 columns x 64 bytes (128 K of fp4)
+// LDS of the K pipeline.  The usual layout: two activation stages, one weight stage (4 KB per wave), the e8m0 scales
+// of the whole tile staged once.  "Ring mode" (fp8 path without the whole-tile scale staging, i.e. pre-shuffled
+// scales, or strided scales that do not fit): the scales of a stage travel with its weights (1 KB per wave and
+// stage), which leaves room for two weight stages and -- for row blocks of at most 64 rows -- three activation
+// stages, so that two stages' copies are in flight instead of one.  The fp8 path needs that: it spends half the
+// matrix-core time per weight byte, and with few rows per expert the stream from HBM is all there is to wait for.
+struct PipeShape {
+  int da, db;        // activation / weight (+ scale) stages
+  int as_bytes;      // block scales of MXFP8 activations: da stages x 4 planes x rows x 4 bytes
+  int scr_bytes;     // ring-mode scale ring: db stages x 4 waves x 1 KB
+  int bytes;
+};
+constexpr PipeShape pipe_shape(bool fp8, bool ring, int lds_rows) {
+  PipeShape p{};
+  p.da = ring && lds_rows <= 64 ? 3 : 2;
+  p.db = ring ? 2 : 1;
+  p.as_bytes = fp8 ? p.da * 4 * (lds_rows < 64 ? 64 : lds_rows) * 4 : 0;
+  p.scr_bytes = ring ? p.db * 4 * 1024 : 0;
+  p.bytes = p.da * lds_rows * 128 + p.db * B_BYTES + p.as_bytes + p.scr_bytes;
+  return p;
+}
 
 // Epilogue of one output tile (shared by every tiled kernel).  The accumulators hold, for fragment
 // (i, f), element j: row 32i + 8(j/4) + 4h + j%4, column t.n0 + wave*64 + c32*NF + f.
@@ -518,6 +539,10 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   constexpr int ESZ = FP8 ? 1 : 2;            // bytes per activation element
   constexpr int KA = A_ROW_BYTES / ESZ;       // K per activation stage
   constexpr int A_STAGE = LDS_ROWS * A_ROW_BYTES;
+  constexpr bool RING = FP8 && !SC_LDS;
+  constexpr PipeShape PS = pipe_shape(FP8, RING, LDS_ROWS);
+  constexpr int DA = PS.da, DB = PS.db;
+  auto a_slot = [](int it) { return DA == 2 ? (it & 1) : it % DA; };
   constexpr uint32_t kOob = 0x7FFFFFFFu;
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -531,13 +556,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
   const uint8_t *s_base = a.w_mx_scale + (int64_t)t.expert * a.w_mx_stride_e;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-  const uint32_t lds_b = lds_base + 2 * A_STAGE + wave * 4096;
-  const uint8_t *bbuf = lds + 2 * A_STAGE + wave * 4096;
+  const uint32_t lds_b = lds_base + DA * A_STAGE + wave * 4096;
+  const uint8_t *bbuf = lds + DA * A_STAGE + wave * 4096;
   // activation block scales (fp8 path): two stages of four planes (one per 32-K group of the stage) of one dword
   // per row; a copy always writes 64 dwords (lanes past the tile's rows write zeros)
   constexpr int AS_ROWS = LDS_ROWS < 64 ? 64 : LDS_ROWS;
-  constexpr int AS_BYTES = FP8 ? 2 * 4 * AS_ROWS * 4 : 0;
-  uint8_t *lds_sc = lds + 2 * A_STAGE + B_BYTES + AS_BYTES;
+  constexpr int AS_BYTES = PS.as_bytes;
+  uint8_t *lds_sc = lds + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
 
   // ---- scales of the whole tile, once.  Strided: 256 columns x G bytes, contiguous in memory.  CDNA4
   // pre-shuffle: the tile's 8 blocks of 32 columns are contiguous too (KSP*32 bytes each); byte
@@ -554,7 +579,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       // by DMA, 1 KB per instruction: in flight together with the first activation / weight stages and
       // awaited with them at the first barrier of the K loop
       const v4i_t rs = make_rsrc(sc_src, (uint32_t)sc_avail);
-      const uint32_t lds_sc_addr = lds_base + 2 * A_STAGE + B_BYTES + AS_BYTES;
+      const uint32_t lds_sc_addr = lds_base + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
       for (int i = wave; i * 1024 < sc_tile_bytes; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
     } else {
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
@@ -596,8 +621,8 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   // LDS, one byte-sized copy per group (64 rows per instruction, waves 0 and 1; groups past K/32 are not read at
   // all, so nothing beyond a row's own scales is touched)
   const bool x_mx = FP8 && a.x_mx_scale != nullptr;
-  const uint32_t lds_as = lds_base + 2 * A_STAGE + B_BYTES;
-  const uint32_t *as_buf = (const uint32_t *)(lds + 2 * A_STAGE + B_BYTES);
+  const uint32_t lds_as = lds_base + DA * A_STAGE + DB * B_BYTES;
+  const uint32_t *as_buf = (const uint32_t *)(lds + DA * A_STAGE + DB * B_BYTES);
   v4i_t ras = rx;
   uint32_t as_off = kOob;
   if (x_mx) {
@@ -614,7 +639,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     if (x_mx && wave * 64 < LDS_ROWS) {
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4)
-        dma1(ras, lds_as + ((it & 1) * 4 + g4) * AS_ROWS * 4 + wave * 256, it * 4 + g4 < G ? as_off : kOob,
+        dma1(ras, lds_as + (a_slot(it) * 4 + g4) * AS_ROWS * 4 + wave * 256, it * 4 + g4 < G ? as_off : kOob,
              (uint32_t)(it * 4 + g4));
     }
   };
@@ -656,20 +681,54 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const int n_ka = (K + KA - 1) / KA;      // activation stages
   const int n_kb = (K + KB - 1) / KB;      // weight super-stages (two activation stages each)
   auto issue_a = [&](int it) {             // clamped: past the end the last stage is copied again
-    it = it < n_ka ? it : n_ka - 1;
+    if constexpr (!RING) it = it < n_ka ? it : n_ka - 1;   // (ring mode: chunks past K are not read at all)
     const int kb = it * KA;
     const uint32_t akill = kb + a_chunk * (16 / ESZ) < K ? 0u : kOob;
-    const uint32_t sb = lds_base + (it & 1) * A_STAGE + wave * 8 * A_ROW_BYTES;
+    const uint32_t sb = lds_base + a_slot(it) * A_STAGE + wave * 8 * A_ROW_BYTES;
 #pragma unroll
     for (int i = 0; i < NFR; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * ESZ);
   };
   auto issue_b = [&](int sup) {
-    sup = sup < n_kb ? sup : n_kb - 1;
+    const uint32_t region = DB == 2 ? (uint32_t)(sup & 1) * B_BYTES : 0u;
+    if constexpr (!RING) sup = sup < n_kb ? sup : n_kb - 1;
     const int kb = sup * KB;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t bkill = (wave_live && kb + w_part[j] * 32 < K) ? 0u : kOob;
-      dma16(rw, lds_b + j * 1024, w_off[j] | bkill, kb >> 1);
+      dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, kb >> 1);
+    }
+  };
+  // ring mode: the scales of weight stage `sup` for this wave's 64 columns, into the wave's 1 KB piece of the scale
+  // ring.  Pre-shuffled layout: one copy -- the wave's two blocks of 32 columns hold the 8 groups that contain the
+  // stage's 4 as 256 contiguous bytes each (lanes 0-15 / 16-31; the other lanes copy nothing).  Strided layout:
+  // one byte-sized copy per group, lane L fetching column L of the strip into dword [group][L]; slow (64 lines
+  // touched per copy) and only used when the scales of a tile do not fit LDS.
+  const uint32_t lds_scr = lds_base + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
+  const uint8_t *scr_buf = lds + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
+  uint32_t scr_voff = kOob;
+  v4i_t rsc = rw;
+  if constexpr (RING) {
+    rsc = make_rsrc(s_base, kOob);
+    if (cdna4) {
+      const int blk = (t.n0 + wave * 64) / 32 + lane / 16;
+      if (lane < 32 && blk * 32 < N && wave_live) scr_voff = (uint32_t)(blk * KSP * 32 + (lane % 16) * 16);
+    } else {
+      const int col = t.n0 + wave * 64 + lane;
+      if (col < N) scr_voff = (uint32_t)((int64_t)col * a.w_mx_stride_n);
+    }
+  }
+  auto issue_sc = [&](int sup) {
+    if constexpr (RING) {
+      const uint32_t dst = lds_scr + ((uint32_t)(sup & 1) * 4 + wave) * 1024;
+      if (cdna4) {
+        dma16(rsc, dst, sup * 4 < G ? scr_voff : kOob, (uint32_t)(256 * (sup >> 1)));
+      } else {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int kg = sup * 4 + g4;
+          dma1(rsc, dst + g4 * 256, kg < G ? scr_voff : kOob, (uint32_t)((int64_t)kg * a.w_mx_stride_k));
+        }
+      }
     }
   };
 
@@ -683,7 +742,8 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int pos = f * 32 + c32;
-        raw[f][q] = *(const uint4 *)(bbuf + pos * 64 + (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
+        raw[f][q] = *(const uint4 *)(bbuf + (DB == 2 ? (sup & 1) * B_BYTES : 0) + pos * 64 +
+                                     (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
         // group kg = 4*sup + 2q + h of this lane's column.  Strided: byte kg, kept inside the column's G bytes
         // (groups past the end of K meet zero codes and zero activations; their scale only has to be some finite
         // value of this column).  Pre-shuffled: byte 256*(kg/8) + 64*(kg%4) + 2*((kg%8)/4); the padding up to a
@@ -692,7 +752,12 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         int kg_off = sup_off + sc_lane_off[q];
         kg_off = kg_off < sc_clamp ? kg_off : sc_clamp;
         uint32_t sbyte;
-        if constexpr (SC_LDS) sbyte = lds_sc[sc_col_off[f] + kg_off];
+        if constexpr (RING) {
+          const uint8_t *piece = scr_buf + ((sup & 1) * 4 + wave) * 1024;
+          const int n = c32 * NF + f;  // column inside the wave's strip
+          sbyte = cdna4 ? piece[(n / 32) * 256 + 64 * (2 * q + h) + 4 * (n % 16) + 2 * (sup & 1) + (n % 32) / 16]
+                        : piece[((2 * q + h) * 64 + n) * 4];
+        } else if constexpr (SC_LDS) sbyte = lds_sc[sc_col_off[f] + kg_off];
         else if (cdna4) sbyte = s_base[sc_col_off[f] + kg_off];
         else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + kg_off];
         if constexpr (FP8) scw[f] = q == 0 ? sbyte : (scw[f] | (sbyte << 8));
@@ -718,13 +783,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   auto fp8_read0 = [&](int it) {
     if constexpr (FP8) {
       if (!wave_live) return;
-      const uint8_t *buf = lds + (it & 1) * A_STAGE;
+      const uint8_t *buf = lds + a_slot(it) * A_STAGE;
       fp8_read_frags(buf, 0, af8[0]);
       // A scale operand: lane half h supplies K block h of an MFMA; byte 0 is the group of s = 0, byte 2 of s = 1
 #pragma unroll
       for (int i = 0; i < NFR; ++i)
-        sa8[i] = x_mx ? (int)(as_buf[((it & 1) * 4 + h) * AS_ROWS + i * 32 + c32] |
-                              (as_buf[((it & 1) * 4 + 2 + h) * AS_ROWS + i * 32 + c32] << 16))
+        sa8[i] = x_mx ? (int)(as_buf[(a_slot(it) * 4 + h) * AS_ROWS + i * 32 + c32] |
+                              (as_buf[(a_slot(it) * 4 + 2 + h) * AS_ROWS + i * 32 + c32] << 16))
                       : 0x7F7F7F7F;
     }
   };
@@ -732,7 +797,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   auto compute = [&](int it, auto qc) {
     constexpr int q = decltype(qc)::value;
     if (!wave_live) return;
-    const uint8_t *buf = lds + (it & 1) * A_STAGE;
+    const uint8_t *buf = lds + a_slot(it) * A_STAGE;
     if constexpr (FP8) {
       // one stage = 128 K = two scaled MFMAs per (row fragment, column fragment); the fragments of the first half
       // and the activations' scale operands are already in registers (fp8_read0)
@@ -778,6 +843,38 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
   };
 
+  if constexpr (RING) {
+    // Stage s requests the activations of stage s + DA - 1 and then the weights and scales of stage s + 2 (the weight
+    // buffer of stage s is free as soon as its contents are in registers).  Copies complete in the order of their
+    // requests, so what may still be in flight at the top of a stage is: with three activation stages, everything the
+    // stage before requested; with two, only the weights and scales it requested (5 copies, or 8 with strided scales).
+    const bool as_wave = x_mx && wave * 64 < LDS_ROWS;
+    constexpr int NSC = 4;  // scale copies of a stage with strided scales (1 when pre-shuffled)
+    if constexpr (DA == 3) {
+      issue_a(0), issue_as(0), issue_b(0), issue_sc(0);
+      issue_a(1), issue_as(1), issue_b(1), issue_sc(1);
+    } else {
+      issue_b(0), issue_sc(0);
+      issue_a(0), issue_as(0), issue_b(1), issue_sc(1);
+    }
+    for (int it = 0; it < n_ka; ++it) {
+      if constexpr (DA == 3) {
+        if (cdna4) { if (as_wave) wait_vmcnt<NFR + 4 + 4 + 1>(); else wait_vmcnt<NFR + 4 + 1>(); }
+        else { if (as_wave) wait_vmcnt<NFR + 4 + 4 + NSC>(); else wait_vmcnt<NFR + 4 + NSC>(); }
+      } else {
+        if (cdna4) wait_vmcnt<4 + 1>(); else wait_vmcnt<4 + NSC>();
+      }
+      __syncthreads();
+      load_b(it);
+      fp8_read0(it);
+      issue_a(it + DA - 1);
+      issue_as(it + DA - 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: their buffer may be refilled
+      issue_b(it + 2);
+      issue_sc(it + 2);
+      compute(it, std::integral_constant<int, 0>{});
+    }
+  } else {
   issue_a(0);
   issue_b(0);
   if constexpr (FP8) {
@@ -811,6 +908,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         compute(it + 1, std::integral_constant<int, 1>{});
       }
     }
+  }
   }
   wait_dma();
 
@@ -858,21 +956,24 @@ __global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a,
 template <int XDT, int BM, int ACT>
 int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int LDS_ROWS = TileShape<XDT, BM>::LDS_ROWS;
-  constexpr int PIPE_BYTES = 2 * LDS_ROWS * A_ROW_BYTES + B_BYTES + (is_fp8(XDT) ? 2 * 4 * (LDS_ROWS < 64 ? 64 : LDS_ROWS) * 4 : 0);
+  constexpr int PIPE_BYTES = pipe_shape(is_fp8(XDT), false, LDS_ROWS).bytes;
+  constexpr int RING_BYTES = pipe_shape(is_fp8(XDT), true, LDS_ROWS).bytes;
   constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
   int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
   int64_t total = (int64_t)grid_m * grid_n;
   if (total <= 0) return 0;
   int64_t launch = ((total + 7) / 8) * 8;
   if (launch > 0x7FFFFFFF) return TAMD_E_UNSUPPORTED;
-  // scales of a tile are staged in LDS when they are dense ([N][K/32]) or pre-shuffled and two workgroups still fit a CU
+  // scales of a tile are staged in LDS when they are dense ([N][K/32]) or pre-shuffled and two workgroups still fit a CU;
+  // the fp8 path does not stage pre-shuffled scales: they travel with the weight stages (ring mode), as strided ones
+  // do when a tile's worth does not fit
   const int64_t G = a.K / 32;
   const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
   const int64_t sc_bytes = (BLOCK_N * (cdna4 ? (G + 7) / 8 * 8 : G) + 1023) / 1024 * 1024;  // whole 1 KB copies
   const bool dense_sc = cdna4 || (a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
                                   aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0);
-  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024;
-  size_t lds_bytes = PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
+  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024 && !(is_fp8(XDT) && cdna4);
+  size_t lds_bytes = is_fp8(XDT) && !sc_in_lds ? RING_BYTES : PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
   if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;
   void (*kern)(tamd_matmul_args, int, int64_t, int);
   if constexpr (is_fp8(XDT))

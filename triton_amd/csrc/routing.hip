@@ -53,16 +53,15 @@ TAMD_DEVICE float group_max_f32(float v) {
   return v;
 }
 
-// L lanes cooperate on one row; EPL > 0 keeps ceil(n_cols/L) <= EPL keys in registers.
+// L lanes cooperate on one row; EPL > 0 keeps ceil(n_cols/L) <= EPL keys in registers.  `row` is the row of this
+// thread's group of L lanes (any row >= n_rows: a group that only takes part in the shuffles); lds_indx, when given,
+// also receives the picked columns ([row][k] ints) for a kernel that goes on to use them.
 template <int DT, int L, int EPL>
-__global__ __launch_bounds__(256) void topk_kernel(const void *__restrict__ x, int64_t x_stride, int n_rows,
-                                                   int n_cols, int k, int apply_softmax, int use_provided,
-                                                   void *__restrict__ y_vals, int16_t *__restrict__ y_indx,
-                                                   int64_t y_stride, uint32_t *__restrict__ bits,
-                                                   int64_t bits_stride_row, int64_t bits_stride_word) {
-  constexpr int ROWS_PER_BLOCK = 256 / L;
+TAMD_DEVICE void topk_row(const void *__restrict__ x, int64_t x_stride, int n_rows, int n_cols, int k,
+                          int apply_softmax, int use_provided, void *__restrict__ y_vals,
+                          int16_t *__restrict__ y_indx, int64_t y_stride, uint32_t *__restrict__ bits,
+                          int64_t bits_stride_row, int64_t bits_stride_word, int64_t row, int32_t *lds_indx) {
   const int sub = threadIdx.x % L;
-  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / L;
   const bool live = row < n_rows;
   const int64_t rrow = live ? row : 0;
   const int64_t xoff = rrow * x_stride;
@@ -111,6 +110,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const void *__restrict__ x, i
   if (live && slot) {
     store_from_f32<DT>(y_vals, rrow * y_stride + sub, v);
     if (!use_provided) y_indx[rrow * y_stride + sub] = (int16_t)my_idx;
+    if (lds_indx) lds_indx[rrow * k + sub] = my_idx;
   }
   const int n_words = (n_cols + 31) / 32;
   const int base_lane = (threadIdx.x % kWave) - sub;
@@ -123,6 +123,17 @@ __global__ __launch_bounds__(256) void topk_kernel(const void *__restrict__ x, i
     }
     if (live && w < n_words) bits[rrow * bits_stride_row + (int64_t)w * bits_stride_word] = word;
   }
+}
+
+template <int DT, int L, int EPL>
+__global__ __launch_bounds__(256) void topk_kernel(const void *__restrict__ x, int64_t x_stride, int n_rows,
+                                                   int n_cols, int k, int apply_softmax, int use_provided,
+                                                   void *__restrict__ y_vals, int16_t *__restrict__ y_indx,
+                                                   int64_t y_stride, uint32_t *__restrict__ bits,
+                                                   int64_t bits_stride_row, int64_t bits_stride_word) {
+  constexpr int ROWS_PER_BLOCK = 256 / L;
+  topk_row<DT, L, EPL>(x, x_stride, n_rows, n_cols, k, apply_softmax, use_provided, y_vals, y_indx, y_stride, bits,
+                       bits_stride_row, bits_stride_word, (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / L, nullptr);
 }
 
 template <int DT>
@@ -445,13 +456,12 @@ __global__ __launch_bounds__(1024) void scan_ragged_kernel(int E, int n_blocks, 
 // For index arrays small enough that the per-chunk histogram fits LDS (n/64 * E ints): histogram,
 // the three prefix sums, the ordering and the ragged tables without leaving the workgroup --
 // one launch instead of four, which is what the cost of routing is made of at these sizes.
-__global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict__ indx, int is16, int n, int E, int k,
-                                                          int nbits, int NC, int P, int32_t *__restrict__ col_sum,
-                                                          int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
-                                                          int32_t *__restrict__ gather, int32_t *__restrict__ offs,
-                                                          int64_t offs_pitch, int32_t *__restrict__ sched,
-                                                          int64_t sched_pitch, int max_blocks) {
-  extern __shared__ int32_t sm[];
+// lidx: the index array in LDS (a kernel that has just computed it), or null to read `indx` from memory.
+TAMD_DEVICE void meta_fused_body(int32_t *sm, const int32_t *lidx, const void *__restrict__ indx, int is16, int n, int E,
+                                 int k, int nbits, int NC, int P, int32_t *__restrict__ col_sum,
+                                 int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
+                                 int32_t *__restrict__ gather, int32_t *__restrict__ offs, int64_t offs_pitch,
+                                 int32_t *__restrict__ sched, int64_t sched_pitch, int max_blocks) {
   int32_t *hist = sm;                         // [NC][E]  counts, then exclusive prefix over chunks
   int32_t *csum = hist + (int64_t)NC * E;     // [E]
   int32_t *coff = csum + E;                   // [E]
@@ -468,7 +478,7 @@ __global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int i = (c0 + 16 * u) * 64 + lane;
-      ev[u] = (c0 + 16 * u < NC && i < n) ? load_indx(indx, is16, i) : -1;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? (lidx ? lidx[i] : load_indx(indx, is16, i)) : -1;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -522,7 +532,7 @@ __global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int i = (c0 + 16 * u) * 64 + lane;
-      ev[u] = (c0 + 16 * u < NC && i < n) ? load_indx(indx, is16, i) : -1;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? (lidx ? lidx[i] : load_indx(indx, is16, i)) : -1;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -550,6 +560,69 @@ __global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict
   ragged_scan_rows(csum, E, tab, offs, offs_pitch);
   __syncthreads();
   ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, 0, 5 * (int64_t)max_blocks);
+}
+
+__global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict__ indx, int is16, int n, int E, int k,
+                                                          int nbits, int NC, int P, int32_t *__restrict__ col_sum,
+                                                          int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
+                                                          int32_t *__restrict__ gather, int32_t *__restrict__ offs,
+                                                          int64_t offs_pitch, int32_t *__restrict__ sched,
+                                                          int64_t sched_pitch, int max_blocks) {
+  extern __shared__ int32_t sm[];
+  meta_fused_body(sm, nullptr, indx, is16, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs, offs_pitch,
+                  sched, sched_pitch, max_blocks);
+}
+
+// ---------------------------------------------------------------------------
+// top-k and all routing metadata in one workgroup (decode sizes)
+// ---------------------------------------------------------------------------
+// With a few dozen tokens the two launches of routing cost more than their work.  Here the 1024 threads first pick
+// the experts of 1024 / L rows at a time (the picked columns also go to LDS), then run the metadata phases of
+// meta_fused_kernel on the index array in LDS.
+template <int DT, int L, int EPL>
+__global__ __launch_bounds__(1024) void routing_fused_kernel(const void *__restrict__ x, int64_t x_stride, int n_rows,
+                                                             int E, int k, void *__restrict__ y_vals,
+                                                             int16_t *__restrict__ y_indx, uint32_t *__restrict__ bits,
+                                                             int64_t bits_stride_row, int64_t bits_stride_word, int nbits,
+                                                             int NC, int P, int32_t *__restrict__ col_sum,
+                                                             int32_t *__restrict__ col_sorted,
+                                                             int32_t *__restrict__ row_sorted, int32_t *__restrict__ gather,
+                                                             int32_t *__restrict__ offs, int64_t offs_pitch,
+                                                             int32_t *__restrict__ sched, int64_t sched_pitch,
+                                                             int max_blocks) {
+  extern __shared__ int32_t sm[];
+  const int n = n_rows * k;
+  int32_t *lidx = sm;                        // [n] picked columns
+  int32_t *meta = sm + (n + 3) / 4 * 4;
+  constexpr int ROWS = 1024 / L;
+  for (int row0 = 0; row0 < n_rows; row0 += ROWS)
+    topk_row<DT, L, EPL>(x, x_stride, n_rows, E, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row, bits_stride_word,
+                         (int64_t)row0 + threadIdx.x / L, lidx);
+  __syncthreads();
+  meta_fused_body(meta, lidx, nullptr, 0, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs, offs_pitch,
+                  sched, sched_pitch, max_blocks);
+}
+
+template <int DT>
+int launch_routing_fused(const void *x, int64_t xs, int n_rows, int E, int k, void *yv, int16_t *yi, uint32_t *bits,
+                         int64_t bsr, int64_t bsw, int nbits, int NC, int P, size_t lds, int32_t *col_sum,
+                         int32_t *col_sorted, int32_t *row_sorted, int32_t *gather, int32_t *offs, int64_t offs_pitch,
+                         int32_t *sched, int64_t sched_pitch, int max_blocks, hipStream_t st) {
+  int need = (E + 7) / 8;
+  if (need < k) need = k;
+#define TAMD_RF(LL, EE)                                                                                              \
+  do {                                                                                                               \
+    auto kern = routing_fused_kernel<DT, LL, EE>;                                                                    \
+    if (int rc = raise_lds_limit_once((const void *)kern)) return rc;                                                \
+    kern<<<1, 1024, lds, st>>>(x, xs, n_rows, E, k, yv, yi, bits, bsr, bsw, nbits, NC, P, col_sum, col_sorted,        \
+                               row_sorted, gather, offs, offs_pitch, sched, sched_pitch, max_blocks);                \
+  } while (0)
+  if (need <= 8) TAMD_RF(8, 8);
+  else if (need <= 16) TAMD_RF(16, 8);
+  else if (need <= 32) TAMD_RF(32, 8);
+  else TAMD_RF(64, 8);
+#undef TAMD_RF
+  return launch_status();
 }
 
 }  // namespace tamd
@@ -693,6 +766,34 @@ extern "C" int tamd_routing(const void *logits, int dtype, int64_t stride, int n
                             int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx, int32_t *gather_indx,
                             int32_t *offs, int64_t offs_pitch, int32_t *schedule, int64_t sched_pitch, int max_n_blocks,
                             int32_t *workspace, void *stream) {
+  // a few rows (at most two passes of the workgroup's 1024 threads over them), at most 512 columns, and the
+  // metadata workspace of one workgroup fits LDS: one launch for everything
+  if (n_rows > 0 && n_cols > 0 && n_cols <= 512 && k >= 1 && k <= 64 && k <= n_cols && logits && y_vals && y_indx && bits &&
+      (dtype == TAMD_F32 || dtype == TAMD_BF16 || dtype == TAMD_F16) && col_sum && offs && col_sorted_indx &&
+      row_sorted_indx && max_n_blocks >= 0 && offs_pitch >= n_cols + 1 && sched_pitch >= max_n_blocks &&
+      (max_n_blocks == 0 || schedule)) {
+    int need = (n_cols + 7) / 8;
+    if (need < k) need = k;
+    const int L = need <= 8 ? 8 : (need <= 16 ? 16 : (need <= 32 ? 32 : 64));
+    const int64_t n = (int64_t)n_rows * k;
+    const int64_t NC = (n + 63) / 64;
+    int64_t P = 1024 / n_cols;
+    P = P < 1 ? 1 : (P > NC ? NC : P);
+    const int64_t ints = (n + 3) / 4 * 4 + NC * n_cols + 2 * (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1) + 17;
+    if (n_rows <= 2 * (1024 / L) && NC <= 64 && ints * 4 <= 156 * 1024) {
+      int nbits = 0;
+      while ((1 << nbits) < n_cols) ++nbits;
+      hipStream_t st = (hipStream_t)stream;
+#define TAMD_RFD(DT)                                                                                                  \
+  return launch_routing_fused<DT>(logits, stride, n_rows, n_cols, k, y_vals, y_indx, bits, bits_stride_row,            \
+                                  bits_stride_word, nbits, (int)NC, (int)P, (size_t)ints * 4, col_sum, col_sorted_indx,  \
+                                  row_sorted_indx, gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, st)
+      if (dtype == TAMD_F32) TAMD_RFD(TAMD_F32);
+      if (dtype == TAMD_BF16) TAMD_RFD(TAMD_BF16);
+      TAMD_RFD(TAMD_F16);
+#undef TAMD_RFD
+    }
+  }
   const int rc = tamd_topk_forward(logits, dtype, stride, n_rows, n_cols, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row,
                                    bits_stride_word, stream);
   if (rc != 0) return rc;
