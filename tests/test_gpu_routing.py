@@ -123,9 +123,12 @@ def test_ragged_metadata(n_slices, device):
     assert torch.equal(m.block_schedule_data.cpu(), ref.block_schedule_data)
 
 
-@pytest.mark.parametrize("T,E,k", [(4096, 128, 4), (64, 128, 4), (16384, 32, 4), (300, 200, 8), (1, 128, 4)])
+@pytest.mark.parametrize("T,E,k", [(4096, 128, 4), (64, 128, 4), (16384, 32, 4), (300, 200, 8), (1, 128, 4), (128, 128, 4),
+                                   (129, 128, 4), (100, 13, 1), (33, 512, 8), (64, 200, 8), (16, 64, 64), (255, 40, 2)])
 def test_routing_configs(T, E, k, device):
-    """BASELINE config 2 (T=4096, E=128, k=4) and the routing of configs 4 / 5, plus a run with exact ties."""
+    """BASELINE config 2 (T=4096, E=128, k=4) and the routing of configs 4 / 5, plus a run with exact ties.  The small
+    row counts run as one launch (top-k and metadata in one workgroup, at most two passes of its 1024 threads over the
+    rows: up to 256, 128, 64 or 32 rows for up to 64, 128, 256 or 512 experts); the cases sit on both sides of that."""
     torch.manual_seed(0)
     for ties in (False, True):
         logits = torch.randn(T, E)
