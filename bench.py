@@ -724,10 +724,14 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: leave out the short runs of the other configurations")
     ap.add_argument("--block-m", type=int, default=0)
-    ap.add_argument("--scale-layout", default="strided", choices=["strided", "cdna4"],
+    ap.add_argument("--scale-layout", default=None, choices=["strided", "cdna4"],
                     help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
-                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout()))")
+                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout())).  Default: strided, except for "
+                    "--workload mlp, which hands over the pre-shuffled scales as the reference's bench_mlp does on this "
+                    "target (make_default_matmul_mxfp4_w_scale_layout, tensor_details/layout.py:43-54)")
     args = ap.parse_args()
+    if args.scale_layout is None:
+        args.scale_layout = "cdna4" if args.workload == "mlp" else "strided"
     args.cpu_work = 1.0
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (with more GPUs the experts "

@@ -234,6 +234,33 @@ def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, fp8, device):
     check(out, ref.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("block_m", [32, 64, 128])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float8_e4m3fn])
+def test_fp8_ragged_long_k_strided_scales(block_m, out_dtype, device):
+    """K = 4608 with strided scales: a tile's scales (256 columns x 144 bytes) no longer fit LDS beside the pipeline of a
+    128-row block, so they travel with the weight stages (byte-sized copies); smaller blocks still stage them.  Also the
+    plain float8_e4m3fn output of fp8-row kernels (the rows the next matmul of a layer consumes)."""
+    torch.manual_seed(3)
+    E, K, N, M = 3, 4608, 264, 300
+    sizes = torch.tensor([130, 0, 170], dtype=torch.int32)
+    x8, xs = to_fp8(torch.randn(M, K), torch.float8_e4m3fn)
+    w = torch.randn(E, K, N) * 0.02
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    gammas = 2.0**torch.randint(-3, 0, (M, )).float()
+    with scoped_opt_flags_constraints({"block_m": block_m}):
+        out = matmul(x8.to(device), v, bias.to(device), md, gammas=gammas.to(device),
+                     precision_config=fp8_pc(s, xs, device, out_dtype, torch.float8_e4m3fn))
+    ref = MR.matmul_ref(x8, rv, bias, slice_sizes=sizes, b_mx_scale=rs, a_flex_scale=xs, gammas=gammas)
+    assert out.dtype == out_dtype
+    if out_dtype == torch.bfloat16:
+        check(out, ref.to(torch.bfloat16))
+    else:
+        # one fp8 step (2^-3 relative) around the float32 result
+        torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=0.0725, atol=2e-2)
+
+
 def test_moe_down_projection_and_combine_small(device):
     """Config-5-shaped pipeline at reduced size: expert-sorted fp8 rows -> grouped GEMM * gate weights ->
     scatter to (token, slot) order -> top-k combine."""

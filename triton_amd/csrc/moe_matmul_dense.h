@@ -146,7 +146,7 @@ TAMD_DEVICE void run_tile_w16(const tamd_matmul_args &a, const Tile &t, uint8_t 
     rd = rd == 2 ? 0 : rd + 1;
   }
   wait_dma();
-  tile_epilogue<NFR, ACT, XDT>(a, t, acc, lds);
+  tile_epilogue<NFR, ACT, XDT, false>(a, t, acc, lds);
 }
 
 template <int XDT, int BM, int ACT, bool WKC>

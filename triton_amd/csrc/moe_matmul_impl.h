@@ -293,6 +293,11 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
   auto narrow = [&](float v) -> uint32_t {  // one output value as 8 / 16 bits
     return ydt == TAMD_BF16 ? f32_to_bf16_bits(v) : (ydt == TAMD_F16 ? f32_to_f16_bits(v) : f32_to_fp8_bits(v, ydt));
   };
+  auto narrow2 = [&](float lo, float hi) -> uint32_t {  // two 16-bit outputs in one word (one packed conversion)
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    if (ydt == TAMD_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, f16x2_t));
+  };
   // without per-row factors bias * beta * out_alpha is one value per column
   float bias_a[NF];
 #pragma unroll
@@ -337,17 +342,13 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
       if constexpr (ROWSC) {
         // the factors of row 32 i + l sit in lane l: lanes of half h need l = 8 (j / 4) + 4 h + j % 4
         const int l0 = (j >> 2) * 8 + (j & 3);
-        float beta = 1.0f;
-        if (has_beta) {
-          const float b0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0));
-          const float b1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0 + 4));
-          beta = h ? b1 : b0;
-        }
-        if (has_gamma) {
-          const float g0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0));
-          const float g1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0 + 4));
-          gamma = h ? g1 : g0;
-        }
+        // (an absent factor was loaded as 1.0: no branch inside the element loop)
+        const float b0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0));
+        const float b1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(beta_of[i]), l0 + 4));
+        const float beta = h ? b1 : b0;
+        const float g0 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0));
+        const float g1 = bits_to_f32(__builtin_amdgcn_readlane((int)f32_to_bits(gamma_of[i]), l0 + 4));
+        gamma = h ? g1 : g0;
 #pragma unroll
         for (int f = 0; f < NF; ++f) v[f] = __builtin_fmaf(acc[i][f][j], flex, bias_a[f] * beta);
       } else {
@@ -402,7 +403,7 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
       if (staged) {
         uint8_t *dstl = ob + (r * OUT_COLS + wave * 32 * NO + c32 * NO) * osz;
         if (osz == 2) {
-          if constexpr (NO == 2) *(uint32_t *)dstl = narrow(o[0]) | (narrow(o[NO - 1]) << 16);
+          if constexpr (NO == 2) *(uint32_t *)dstl = narrow2(o[0], o[NO - 1]);
           else *(uint16_t *)dstl = (uint16_t)narrow(o[0]);
         } else {
           if constexpr (NO == 2) *(uint16_t *)dstl = (uint16_t)(narrow(o[0]) | (narrow(o[NO - 1]) << 8));
@@ -507,11 +508,15 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
 
 // FAST_YDT: the 16-bit output type that gets the specialised epilogues (the activations' type; bf16 for fp8
 // activations); any other combination takes the general one.
-template <int NFR, int ACT, int FAST_YDT>
+// FP8_ROWS: the kernel's activations are fp8; then a plain float8_e4m3fn output (the rows the next matmul of an
+// MoE layer consumes) is specialised as well.
+template <int NFR, int ACT, int FAST_YDT, bool FP8_ROWS>
 TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const bool flexo = a.y_expected_scale != nullptr || a.y_actual_scale != nullptr;
   if (a.y_mx_scale) {  // always e4m3 values and no flexpoint output (checked by the entry point)
     tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false, true>(a, t, acc, lds);
+  } else if (FP8_ROWS && a.y_dtype == TAMD_FP8_E4M3 && !flexo) {
+    if constexpr (FP8_ROWS) tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false>(a, t, acc, lds);
   } else if (a.y_dtype == FAST_YDT && !flexo) {
     if (a.betas || a.gammas) tile_epilogue_t<NFR, ACT, FAST_YDT, true, false>(a, t, acc, lds);
     else tile_epilogue_t<NFR, ACT, FAST_YDT, false, false>(a, t, acc, lds);
@@ -912,7 +917,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   wait_dma();
 
-  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT>(a, t, acc, lds);
+  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT, FP8>(a, t, acc, lds);
 }
 
 // Row fragments a workgroup can hold: a 128-row block of 16-bit activations also takes a remainder of
