@@ -261,6 +261,34 @@ def test_fp8_ragged_long_k_strided_scales(block_m, out_dtype, device):
         torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=0.0725, atol=2e-2)
 
 
+@pytest.mark.parametrize("kind", ["tiled_bf16", "stream_bf16", "tiled_fp8"])
+def test_zero_scale_bytes_with_nonzero_codes(kind, device):
+    """A checkpoint prepared elsewhere may hold e8m0 bytes of 0 next to non-zero codes (downcast_to_mxfp never writes
+    that).  The reference multiplies such a group by +0.0; the conversion instructions multiply by 2^-127, i.e. the group
+    contributes at most 6 * 2^-127 per element: the outputs agree with the oracle to far below the tolerance."""
+    torch.manual_seed(11)
+    M, K, N = (8, 256, 64) if kind == "stream_bf16" else (150, 256, 264)
+    w = torch.randn(1, K, N) * 0.05
+    v, s, rv, rs = quantize_w(w, device)
+    rs = rs.clone()
+    rs[0, ::3, ::2] = 0          # every third group of every second column
+    s = rs.to(device)
+    assert int((rv[0, :16, 0] != 0).sum()) > 0  # the zeroed groups do hold non-zero codes
+    bias = torch.randn(1, N)
+    sizes = torch.tensor([M], dtype=torch.int32)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    if kind == "tiled_fp8":
+        x8, xs = to_fp8(torch.randn(M, K))
+        out = matmul(x8.to(device), v, bias.to(device), md, precision_config=fp8_pc(s, xs, device, torch.bfloat16))
+        ref = MR.matmul_ref(x8, rv, bias, slice_sizes=sizes, b_mx_scale=rs, a_flex_scale=xs).to(torch.bfloat16)
+    else:
+        x = torch.randn(M, K).to(torch.bfloat16)
+        out = matmul(x.to(device), v, bias.to(device), md, precision_config=PrecisionConfig(b_mx_scale=s, b_microblock_size=32))
+        ref = MR.matmul_ref(x, rv, bias, slice_sizes=sizes, b_mx_scale=rs)
+    assert torch.isfinite(out.float()).all()
+    check(out, ref)
+
+
 def test_moe_down_projection_and_combine_small(device):
     """Config-5-shaped pipeline at reduced size: expert-sorted fp8 rows -> grouped GEMM * gate weights ->
     scatter to (token, slot) order -> top-k combine."""
