@@ -38,7 +38,10 @@ TAMD_DEVICE uint32_t e2m1_word_scaled(const float (&v)[8], float ds) {
   return w;
 }
 
-// 16-byte accesses to memory that is touched once (non-temporal)
+// 16-byte accesses to memory that is touched once (non-temporal).  Measured on the two tile kernels below: the
+// quantiser is fastest with non-temporal loads of its source and ordinary stores of the codes (110 us; 130 with
+// ordinary loads), the dequantiser with ordinary loads of the codes and non-temporal stores of its rows (61 us; 67 with
+// ordinary stores, 71 with both non-temporal).
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 TAMD_DEVICE uint4 load_once(const void *p) {
   u32x4_t q = __builtin_nontemporal_load((const u32x4_t *)p);
@@ -47,6 +50,13 @@ TAMD_DEVICE uint4 load_once(const void *p) {
 TAMD_DEVICE void store_once(void *p, uint4 v) {
   __builtin_nontemporal_store(u32x4_t{v.x, v.y, v.z, v.w}, (u32x4_t *)p);
 }
+// the same as ordinary accesses; through the vector type so that they stay one 16-byte instruction (a 16-byte access
+// through a pointer derived from char * is split into four 4-byte ones otherwise, a quarter of the bandwidth)
+TAMD_DEVICE uint4 load16(const void *p) {
+  u32x4_t q = *(const u32x4_t *)p;
+  return make_uint4(q.x, q.y, q.z, q.w);
+}
+TAMD_DEVICE void store16(void *p, uint4 v) { *(u32x4_t *)p = u32x4_t{v.x, v.y, v.z, v.w}; }
 
 // Value kinds of a microscaled tensor: e2m1 codes (two per byte), or fp8 bytes.  Largest magnitude and
 // largest power of two of each (mxfp.py:206-209, mxfp_details/_downcast_to_mxfp.py:24-31).
@@ -217,8 +227,7 @@ __global__ __launch_bounds__(256) void downcast_cols_kernel(
 // downcast, source contiguous along r, 16-byte aligned: a workgroup quantises a tile of GT groups x 32*NV
 // columns.  A load instruction of a wave reads 512 contiguous bytes of two source rows (a thread keeps the 32
 // rows of its NV columns in registers, as above); the codes pass through LDS so that they leave as GT x 16
-// contiguous bytes per column.  The source is read once and the codes are not read back here: both bypass the
-// caches' retention (non-temporal), which is worth a quarter of the time on this memory system.
+// contiguous bytes per column.  The source is read once: its loads are non-temporal.
 // ---------------------------------------------------------------------------
 // groups per tile: 64 KiB of codes in LDS either way
 template <int DT>
@@ -312,7 +321,7 @@ __global__ __launch_bounds__(256) void downcast_cols_tile_kernel(
   if (part < n_g) {
 #pragma unroll 4
     for (int c = threadIdx.x / GT; c < n_c; c += 256 / GT) {
-      store_once(vbase + (int64_t)c * vsr + part * 16, s_codes[c * GT + (part ^ ((c / NV) & 7))]);
+      store16(vbase + (int64_t)c * vsr + part * 16, s_codes[c * GT + (part ^ ((c / NV) & 7))]);
       sbase[(int64_t)c * csr + part] = s_sc[c * GT + part];
     }
   }
@@ -479,7 +488,7 @@ __global__ __launch_bounds__(256) void upcast_cols_tile_kernel(
   if (part < n_g) {
 #pragma unroll 4
     for (int c = threadIdx.x / GT; c < n_c; c += 256 / GT) {
-      s_codes[c * GT + (part ^ ((c / NV) & 7))] = load_once(vbase + (int64_t)c * vsr + part * 16);
+      s_codes[c * GT + (part ^ ((c / NV) & 7))] = load16(vbase + (int64_t)c * vsr + part * 16);
       s_sc[c * GT + part] = sbase[(int64_t)c * csr + part];
     }
   }
