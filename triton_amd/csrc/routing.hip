@@ -27,30 +27,48 @@ TAMD_DEVICE uint64_t logit_key(float x, int col) {
   return ((uint64_t)u << 16) | (uint64_t)(0xFFFFu - (uint32_t)col);
 }
 
-template <int L>
+// Inverse of the value part of logit_key (a -0.0 logit comes back as +0.0).
+TAMD_DEVICE float logit_of_key(uint64_t key) {
+  uint32_t u = (uint32_t)(key >> 16);
+  u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+  return bits_to_f32(u);
+}
+
+// Step O (1, 2, 4, ...) of a butterfly reduction over groups of lanes: the value of a lane of the other aligned block
+// of O lanes.  All lanes of a block of O hold the same value by then, so for O = 4 and 8 the partner may be the
+// mirrored lane, which, like the swaps inside a quad, the data-parallel move does in the register file; from 16 up it
+// is the lane at XOR distance O, through the LDS crossbar.
+template <int O>
+TAMD_DEVICE uint32_t butterfly_partner(uint32_t v) {
+  if constexpr (O == 1) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);        // quad_perm [1,0,3,2]
+  else if constexpr (O == 2) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+  else if constexpr (O == 4) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+  else if constexpr (O == 8) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);  // row_mirror
+  else return (uint32_t)__shfl_xor((int)v, O);
+}
+
+template <int L, int O = 1>
 TAMD_DEVICE uint64_t group_max_u64(uint64_t v) {
-#pragma unroll
-  for (int o = 1; o < L; o <<= 1) {
-    uint32_t lo = __shfl_xor((uint32_t)v, o);
-    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), o);
-    uint64_t w = ((uint64_t)hi << 32) | lo;
-    v = w > v ? w : v;
+  if constexpr (O < L) {
+    const uint32_t lo = butterfly_partner<O>((uint32_t)v);
+    const uint32_t hi = butterfly_partner<O>((uint32_t)(v >> 32));
+    const uint64_t w = ((uint64_t)hi << 32) | lo;
+    return group_max_u64<L, O * 2>(w > v ? w : v);
+  } else {
+    return v;
   }
-  return v;
 }
 
-template <int L>
+template <int L, int O = 1>
 TAMD_DEVICE float group_sum_f32(float v) {
-#pragma unroll
-  for (int o = 1; o < L; o <<= 1) v += __shfl_xor(v, o);
-  return v;
+  if constexpr (O < L) return group_sum_f32<L, O * 2>(v + bits_to_f32(butterfly_partner<O>(f32_to_bits(v))));
+  else return v;
 }
 
-template <int L>
+template <int L, int O = 1>
 TAMD_DEVICE float group_max_f32(float v) {
-#pragma unroll
-  for (int o = 1; o < L; o <<= 1) v = __builtin_fmaxf(v, __shfl_xor(v, o));
-  return v;
+  if constexpr (O < L) return group_max_f32<L, O * 2>(__builtin_fmaxf(v, bits_to_f32(butterfly_partner<O>(f32_to_bits(v)))));
+  else return v;
 }
 
 // L lanes cooperate on one row; EPL > 0 keeps ceil(n_cols/L) <= EPL keys in registers.  `row` is the row of this
@@ -66,19 +84,30 @@ TAMD_DEVICE void topk_row(const void *__restrict__ x, int64_t x_stride, int n_ro
   const int64_t rrow = live ? row : 0;
   const int64_t xoff = rrow * x_stride;
   int my_idx = 0;
+  uint64_t mine = 0ull;  // key of the column this lane's slot picked
   if (use_provided) {
     if (sub < k) my_idx = y_indx[rrow * y_stride + sub];
   } else {
     uint64_t keys[EPL > 0 ? EPL : 1];
     if constexpr (EPL > 0) {
+      // every lane loads (columns past the end re-read the last one) and the values are pinned before they are
+      // selected: a load that the compiler may move under the per-lane condition is awaited before the next one is
+      // issued, eight round trips to memory instead of one
+      float xv[EPL];
 #pragma unroll
       for (int j = 0; j < EPL; ++j) {
-        int c = sub + j * L;
-        keys[j] = c < n_cols ? logit_key(load_as_f32<DT>(x, xoff + c), c) : 0ull;
+        const int c = sub + j * L;
+        xv[j] = load_as_f32<DT>(x, xoff + (c < n_cols ? c : n_cols - 1));
+      }
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) asm volatile("" : "+v"(xv[j]));
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) {
+        const int c = sub + j * L;
+        keys[j] = c < n_cols ? logit_key(xv[j], c) : 0ull;
       }
     }
     uint64_t prev = ~0ull;
-    uint64_t mine = 0ull;
     for (int pass = 0; pass < k; ++pass) {
       uint64_t best = 0ull;
       if constexpr (EPL > 0) {
@@ -100,7 +129,12 @@ TAMD_DEVICE void topk_row(const void *__restrict__ x, int64_t x_stride, int n_ro
     my_idx = (int)(0xFFFFu - (uint32_t)(mine & 0xFFFFull));
   }
   const bool slot = sub < k;
-  float v = slot ? load_as_f32<DT>(x, xoff + my_idx) : 0.f;
+  float v;
+  if (apply_softmax && !use_provided) {
+    v = slot ? logit_of_key(mine) : 0.f;  // a zero's sign is lost in the key and makes no difference to the softmax
+  } else {
+    v = slot ? load_as_f32<DT>(x, xoff + my_idx) : 0.f;
+  }
   if (apply_softmax) {
     float mx = group_max_f32<L>(slot ? v : -__builtin_inff());
     float e = slot ? expf(v - mx) : 0.f;
@@ -183,15 +217,15 @@ TAMD_DEVICE uint64_t lanemask_lt() {
   return lane == 0 ? 0ull : (~0ull >> (64 - lane));
 }
 
-__global__ __launch_bounds__(256) void hist_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
+__global__ __launch_bounds__(1024) void hist_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
                                                    int CH, int nbits, int32_t *__restrict__ chunk_pref,
                                                    int32_t *__restrict__ block_tot) {
   extern __shared__ int32_t hist[];  // [CH][E]
   const int blk = blockIdx.x;
-  for (int i = threadIdx.x; i < CH * E; i += 256) hist[i] = 0;
+  for (int i = threadIdx.x; i < CH * E; i += 1024) hist[i] = 0;
   __syncthreads();
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  for (int c = wave; c < CH; c += 4) {
+  for (int c = wave; c < CH; c += 16) {  // CH <= 16: one chunk per wave, so a workgroup waits for memory once
     int64_t i = ((int64_t)blk * CH + c) * 64 + lane;
     int e = i < n ? load_indx(indx, is16, i) : -1;
     bool valid = e >= 0 && e < E;
@@ -199,7 +233,7 @@ __global__ __launch_bounds__(256) void hist_kernel(const void *__restrict__ indx
     if (valid && (same & lanemask_lt()) == 0) hist[c * E + e] = __popcll(same);
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < E; e += 256) {
+  for (int e = threadIdx.x; e < E; e += 1024) {
     int run = 0;
     for (int c = 0; c < CH; ++c) {
       int t = hist[c * E + e];
@@ -210,15 +244,22 @@ __global__ __launch_bounds__(256) void hist_kernel(const void *__restrict__ indx
   }
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave (all of them active), in the register file: shifts inside the rows
+// of 16 lanes, then the last lane of rows 0 and 2 added to rows 1 and 3, then lane 31 added to the upper half.
+TAMD_DEVICE int wave_incl_scan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1 (a lane without a source adds 0)
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Exclusive scan of up to 1024 ints held one per thread; returns the total.
 TAMD_DEVICE int block_excl_scan_1024(int v, int &total, int *lds /* >= 17 ints */) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  int inc = v;
-#pragma unroll
-  for (int o = 1; o < kWave; o <<= 1) {
-    int t = __shfl_up(inc, o);
-    if (lane >= o) inc += t;
-  }
+  const int inc = wave_incl_scan(v);
   __syncthreads();
   if (lane == kWave - 1) lds[wave] = inc;
   __syncthreads();
@@ -236,6 +277,28 @@ TAMD_DEVICE int block_excl_scan_1024(int v, int &total, int *lds /* >= 17 ints *
   return inc - v + lds[wave];
 }
 
+// Exclusive prefix over the workgroups' totals of expert e (written to `out` when given; it may be `tot` itself);
+// returns the expert's total.  Sixteen totals are loaded before any of them is used or stored, so that a thread
+// waits for memory once per sixteen blocks and not once per block.
+TAMD_DEVICE int scan_block_totals(const int32_t *tot, int32_t *out, int n_blocks, int E, int e) {
+  int run = 0;
+  for (int b0 = 0; b0 < n_blocks; b0 += 16) {
+    int t[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) t[u] = tot[(int64_t)(b0 + u < n_blocks ? b0 + u : n_blocks - 1) * E + e];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) asm volatile("" : "+v"(t[u]));
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      if (b0 + u < n_blocks) {
+        if (out) out[(int64_t)(b0 + u) * E + e] = run;
+        run += t[u];
+      }
+    }
+  }
+  return run;
+}
+
 __global__ __launch_bounds__(1024) void scan_kernel(int E, int n_blocks, int32_t *__restrict__ block_tot,
                                                     int32_t *__restrict__ col_sum, int32_t *__restrict__ col_offs,
                                                     int32_t *__restrict__ n_valid) {
@@ -245,12 +308,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(int E, int n_blocks, int32_t
     int e = e0 + threadIdx.x;
     int run = 0;
     if (e < E) {
-#pragma unroll 4
-      for (int b = 0; b < n_blocks; ++b) {
-        int t = block_tot[(int64_t)b * E + e];
-        block_tot[(int64_t)b * E + e] = run;
-        run += t;
-      }
+      run = scan_block_totals(block_tot, block_tot, n_blocks, E, e);
       col_sum[e] = run;
     }
     int total;
@@ -261,7 +319,7 @@ __global__ __launch_bounds__(1024) void scan_kernel(int E, int n_blocks, int32_t
   if (threadIdx.x == 0) *n_valid = carry;
 }
 
-__global__ __launch_bounds__(256) void order_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
+__global__ __launch_bounds__(1024) void order_kernel(const void *__restrict__ indx, int is16, int64_t n, int E,
                                                     int CH, int nbits, int k, const int32_t *__restrict__ chunk_pref,
                                                     const int32_t *__restrict__ block_off,
                                                     const int32_t *__restrict__ col_offs,
@@ -271,7 +329,7 @@ __global__ __launch_bounds__(256) void order_kernel(const void *__restrict__ ind
   const int blk = blockIdx.x;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int nv = *n_valid;
-  for (int c = wave; c < CH; c += 4) {
+  for (int c = wave; c < CH; c += 16) {
     int64_t chunk = (int64_t)blk * CH + c;
     int64_t i = chunk * 64 + lane;
     int e = i < n ? load_indx(indx, is16, i) : -1;
@@ -325,12 +383,12 @@ inline int launch_bitmatrix_metadata(const void *indx, int is16, int64_t n, int 
                                      hipStream_t st, bool before_order(void *), void *ctx) {
   MetaPlan p = make_meta_plan(n, E);
   size_t lds = (size_t)p.CH * E * 4;
-  hist_kernel<<<dim3((unsigned)p.n_blocks), 256, lds, st>>>(indx, is16, n, E, p.CH, p.nbits, ws + p.off_chunk_pref,
+  hist_kernel<<<dim3((unsigned)p.n_blocks), 1024, lds, st>>>(indx, is16, n, E, p.CH, p.nbits, ws + p.off_chunk_pref,
                                                            ws + p.off_block_tot);
   scan_kernel<<<1, 1024, 0, st>>>(E, (int)p.n_blocks, ws + p.off_block_tot, col_sum, ws + p.off_col_offs,
                                   ws + p.off_n_valid);
   if (before_order && !before_order(ctx)) return launch_status();
-  order_kernel<<<dim3((unsigned)p.n_blocks), 256, 0, st>>>(indx, is16, n, E, p.CH, p.nbits, k, ws + p.off_chunk_pref,
+  order_kernel<<<dim3((unsigned)p.n_blocks), 1024, 0, st>>>(indx, is16, n, E, p.CH, p.nbits, k, ws + p.off_chunk_pref,
                                                           ws + p.off_block_tot, ws + p.off_col_offs,
                                                           ws + p.off_n_valid, col_sorted, row_sorted, gather);
   return launch_status();
@@ -352,12 +410,7 @@ TAMD_DEVICE void ragged_scan_rows(const int32_t *sizes, int S, int32_t *tab, int
   for (int s0 = 0; s0 < S; s0 += kWave) {
     const int s = s0 + lane;
     const int v = s < S ? ((sizes[s] + ((1 << sh) - 1)) >> sh) : 0;
-    int inc = v;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-      const int t = __shfl_up(inc, o);
-      if (lane >= o) inc += t;
-    }
+    const int inc = wave_incl_scan(v);
     if (s < S) {
       trow[s] = carry + inc - v;
       if (grow) grow[s] = carry + inc - v;
@@ -375,8 +428,10 @@ TAMD_DEVICE void ragged_scan_rows(const int32_t *sizes, int S, int32_t *tab, int
 // the last block.  Entries [first, first + count) of the flattened [5][max_blocks] table.
 TAMD_DEVICE void ragged_fill_schedule(const int32_t *tab, int S, int32_t *sched, int64_t sched_pitch, int max_blocks,
                                       int64_t first, int64_t count) {
+  const bool narrow = first + count <= 0x7FFFFFFF;  // then the table index is found with a 32-bit division
   for (int64_t idx = first + threadIdx.x; idx < first + count; idx += blockDim.x) {
-    const int b = (int)(idx / max_blocks), j = (int)(idx - (int64_t)b * max_blocks);
+    const int b = narrow ? (int)((uint32_t)idx / (uint32_t)max_blocks) : (int)(idx / max_blocks);
+    const int j = (int)(idx - (int64_t)b * max_blocks);
     const int32_t *row = tab + (int64_t)(b + 1) * (S + 1);
     int val = -1;
     if (j < row[S]) {
@@ -425,12 +480,7 @@ __global__ __launch_bounds__(1024) void scan_ragged_kernel(int E, int n_blocks, 
     const int e = e0 + threadIdx.x;
     int run = 0;
     if (e < E) {
-#pragma unroll 4
-      for (int b = 0; b < n_blocks; ++b) {
-        const int t = block_tot[(int64_t)b * E + e];
-        if (lead) block_off[(int64_t)b * E + e] = run;
-        run += t;
-      }
+      run = scan_block_totals(block_tot, lead ? block_off : nullptr, n_blocks, E, e);
       csum[e] = run;
       if (lead) col_sum[e] = run;
     }
@@ -457,28 +507,36 @@ __global__ __launch_bounds__(1024) void scan_ragged_kernel(int E, int n_blocks, 
 // the three prefix sums, the ordering and the ragged tables without leaving the workgroup --
 // one launch instead of four, which is what the cost of routing is made of at these sizes.
 // lidx: the index array in LDS (a kernel that has just computed it), or null to read `indx` from memory.
-TAMD_DEVICE void meta_fused_body(int32_t *sm, const int32_t *lidx, const void *__restrict__ indx, int is16, int n, int E,
-                                 int k, int nbits, int NC, int P, int32_t *__restrict__ col_sum,
+TAMD_DEVICE void meta_fused_body(int32_t *sm, bool zeroed, const int32_t *lidx, const void *__restrict__ indx, int is16,
+                                 int n, int E, int k, int nbits, int NC, int P, int32_t *__restrict__ col_sum,
                                  int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
                                  int32_t *__restrict__ gather, int32_t *__restrict__ offs, int64_t offs_pitch,
                                  int32_t *__restrict__ sched, int64_t sched_pitch, int max_blocks) {
   int32_t *hist = sm;                         // [NC][E]  counts, then exclusive prefix over chunks
   int32_t *csum = hist + (int64_t)NC * E;     // [E]
-  int32_t *coff = csum + E;                   // [E]
-  int32_t *psum = coff + E;                   // [P][E]   partial sums of chunk ranges
+  int32_t *psum = csum + E;                   // [P][E]   partial sums of chunk ranges
   int32_t *tab = psum + (int64_t)P * E;       // [6][E + 1]
-  int32_t *scr = tab + 6 * (E + 1);           // [17]
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
-  for (int i = tid; i < NC * E; i += 1024) hist[i] = 0;
-  __syncthreads();
+  if (!zeroed) {
+    for (int i = tid; i < NC * E; i += 1024) hist[i] = 0;
+    __syncthreads();
+  }
   // 1. per-chunk histogram.  A wave takes its chunks eight at a time so that eight index loads are in
   // flight together (one workgroup has nothing else to hide their latency with).
-  for (int c0 = wave; c0 < NC; c0 += 16 * 8) {
+  for (int c0 = wave; c0 < NC && n > 0; c0 += 16 * 8) {
     int ev[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {  // unconditional loads (entries past the end re-read entry 0), so all eight are in flight
+      const int i = (c0 + 16 * u) * 64 + lane;
+      const bool ok = c0 + 16 * u < NC && i < n;
+      ev[u] = lidx ? lidx[ok ? i : 0] : load_indx(indx, is16, ok ? i : 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) asm volatile("" : "+v"(ev[u]));  // pinned: the loads stay outside the selection below
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int i = (c0 + 16 * u) * 64 + lane;
-      ev[u] = (c0 + 16 * u < NC && i < n) ? (lidx ? lidx[i] : load_indx(indx, is16, i)) : -1;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? ev[u] : -1;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -491,8 +549,20 @@ TAMD_DEVICE void meta_fused_body(int32_t *sm, const int32_t *lidx, const void *_
     }
   }
   __syncthreads();
-  // 2. exclusive prefix over chunks for every expert: P chunk ranges per expert, two passes
+  // 2. exclusive prefix over chunks for every expert: a few chunks in one go, else P chunk ranges per expert in two passes
   const int per = (NC + P - 1) / P;
+  if (NC <= 8) {
+    for (int e = tid; e < E; e += 1024) {
+      int run = 0;
+      for (int c = 0; c < NC; ++c) {
+        const int v = hist[c * E + e];
+        hist[c * E + e] = run;
+        run += v;
+      }
+      csum[e] = run;
+      col_sum[e] = run;
+    }
+  } else {
   for (int t = tid; t < P * E; t += 1024) {
     const int part = t / E, e = t - part * E;
     int run = 0;
@@ -514,25 +584,28 @@ TAMD_DEVICE void meta_fused_body(int32_t *sm, const int32_t *lidx, const void *_
       col_sum[e] = run;
     }
   }
-  __syncthreads();
-  // 3. exclusive prefix over experts
-  int carry = 0;
-  for (int e0 = 0; e0 < E; e0 += 1024) {
-    const int e = e0 + tid;
-    int total;
-    const int ex = block_excl_scan_1024(e < E ? csum[e] : 0, total, scr);
-    if (e < E) coff[e] = carry + ex;
-    carry += total;
-    __syncthreads();
   }
-  const int nv = carry;
+  __syncthreads();
+  // 3. ragged tables of the histogram; the first one is the exclusive prefix over experts that places the entries
+  ragged_scan_rows(csum, E, tab, offs, offs_pitch);
+  __syncthreads();
+  const int32_t *coff = tab;
+  const int nv = tab[E];
   // 4. placement
-  for (int c0 = wave; c0 < NC; c0 += 16 * 8) {
+  for (int c0 = wave; c0 < NC && n > 0; c0 += 16 * 8) {
     int ev[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {  // unconditional loads (entries past the end re-read entry 0), so all eight are in flight
+      const int i = (c0 + 16 * u) * 64 + lane;
+      const bool ok = c0 + 16 * u < NC && i < n;
+      ev[u] = lidx ? lidx[ok ? i : 0] : load_indx(indx, is16, ok ? i : 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) asm volatile("" : "+v"(ev[u]));  // pinned: the loads stay outside the selection below
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int i = (c0 + 16 * u) * 64 + lane;
-      ev[u] = (c0 + 16 * u < NC && i < n) ? (lidx ? lidx[i] : load_indx(indx, is16, i)) : -1;
+      ev[u] = (c0 + 16 * u < NC && i < n) ? ev[u] : -1;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -556,9 +629,7 @@ TAMD_DEVICE void meta_fused_body(int32_t *sm, const int32_t *lidx, const void *_
       }
     }
   }
-  // 5. ragged tables of the histogram
-  ragged_scan_rows(csum, E, tab, offs, offs_pitch);
-  __syncthreads();
+  // 5. block schedule (reads the tables only: no barrier after the placement)
   ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, 0, 5 * (int64_t)max_blocks);
 }
 
@@ -569,8 +640,8 @@ __global__ __launch_bounds__(1024) void meta_fused_kernel(const void *__restrict
                                                           int64_t offs_pitch, int32_t *__restrict__ sched,
                                                           int64_t sched_pitch, int max_blocks) {
   extern __shared__ int32_t sm[];
-  meta_fused_body(sm, nullptr, indx, is16, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs, offs_pitch,
-                  sched, sched_pitch, max_blocks);
+  meta_fused_body(sm, false, nullptr, indx, is16, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs,
+                  offs_pitch, sched, sched_pitch, max_blocks);
 }
 
 // ---------------------------------------------------------------------------
@@ -595,12 +666,13 @@ __global__ __launch_bounds__(1024) void routing_fused_kernel(const void *__restr
   int32_t *lidx = sm;                        // [n] picked columns
   int32_t *meta = sm + (n + 3) / 4 * 4;
   constexpr int ROWS = 1024 / L;
+  for (int i = threadIdx.x; i < NC * E; i += 1024) meta[i] = 0;  // the histograms (the barrier below covers them)
   for (int row0 = 0; row0 < n_rows; row0 += ROWS)
     topk_row<DT, L, EPL>(x, x_stride, n_rows, E, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row, bits_stride_word,
                          (int64_t)row0 + threadIdx.x / L, lidx);
   __syncthreads();
-  meta_fused_body(meta, lidx, nullptr, 0, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs, offs_pitch,
-                  sched, sched_pitch, max_blocks);
+  meta_fused_body(meta, true, lidx, nullptr, 0, n, E, k, nbits, NC, P, col_sum, col_sorted, row_sorted, gather, offs,
+                  offs_pitch, sched, sched_pitch, max_blocks);
 }
 
 template <int DT>
@@ -719,7 +791,7 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
     const int64_t NC = (n_indx + 63) / 64 > 0 ? (n_indx + 63) / 64 : 1;
     int64_t P = 1024 / n_cols;
     P = P < 1 ? 1 : (P > NC ? NC : P);
-    const int64_t ints = NC * n_cols + 2 * (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1) + 17;
+    const int64_t ints = NC * n_cols + (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1);
     if (NC <= 64 && ints * 4 <= 156 * 1024) {  // beyond ~4096 entries one CU is slower than three launches
       int nbits = 0;
       while ((1 << nbits) < n_cols) ++nbits;
@@ -735,7 +807,7 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
     // three launches: histograms per workgroup, scans + ragged tables, placement
     hipStream_t st = (hipStream_t)stream;
     MetaPlan p = make_meta_plan(n_indx, n_cols);
-    hist_kernel<<<dim3((unsigned)p.n_blocks), 256, (size_t)p.CH * n_cols * 4, st>>>(
+    hist_kernel<<<dim3((unsigned)p.n_blocks), 1024, (size_t)p.CH * n_cols * 4, st>>>(
         indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, workspace + p.off_chunk_pref, workspace + p.off_block_tot);
     if (int rc = raise_lds_limit_once((const void *)scan_ragged_kernel)) return rc;
     int64_t wgs = (5 * (int64_t)max_n_blocks + 4095) / 4096;
@@ -743,7 +815,7 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
     scan_ragged_kernel<<<dim3((unsigned)wgs), 1024, sr_lds, st>>>(
         n_cols, (int)p.n_blocks, workspace + p.off_block_tot, workspace + p.off_block_off, col_sum,
         workspace + p.off_col_offs, workspace + p.off_n_valid, offs, offs_pitch, schedule, sched_pitch, max_n_blocks);
-    order_kernel<<<dim3((unsigned)p.n_blocks), 256, 0, st>>>(
+    order_kernel<<<dim3((unsigned)p.n_blocks), 1024, 0, st>>>(
         indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, k, workspace + p.off_chunk_pref, workspace + p.off_block_off,
         workspace + p.off_col_offs, workspace + p.off_n_valid, col_sorted_indx, row_sorted_indx, gather_indx);
     return launch_status();
@@ -779,7 +851,7 @@ extern "C" int tamd_routing(const void *logits, int dtype, int64_t stride, int n
     const int64_t NC = (n + 63) / 64;
     int64_t P = 1024 / n_cols;
     P = P < 1 ? 1 : (P > NC ? NC : P);
-    const int64_t ints = (n + 3) / 4 * 4 + NC * n_cols + 2 * (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1) + 17;
+    const int64_t ints = (n + 3) / 4 * 4 + NC * n_cols + (int64_t)n_cols + P * n_cols + 6 * (int64_t)(n_cols + 1);
     if (n_rows <= 2 * (1024 / L) && NC <= 64 && ints * 4 <= 156 * 1024) {
       int nbits = 0;
       while ((1 << nbits) < n_cols) ++nbits;
