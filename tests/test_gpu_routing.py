@@ -124,11 +124,16 @@ def test_ragged_metadata(n_slices, device):
 
 
 @pytest.mark.parametrize("T,E,k", [(4096, 128, 4), (64, 128, 4), (16384, 32, 4), (300, 200, 8), (1, 128, 4), (128, 128, 4),
-                                   (129, 128, 4), (100, 13, 1), (33, 512, 8), (64, 200, 8), (16, 64, 64), (255, 40, 2)])
+                                   (129, 128, 4), (100, 13, 1), (33, 512, 8), (64, 200, 8), (16, 64, 64), (255, 40, 2),
+                                   (8192, 128, 4), (8193, 128, 4), (4000, 128, 4), (1000, 100, 3), (500, 200, 3),
+                                   (2000, 400, 4), (3000, 64, 8)])
 def test_routing_configs(T, E, k, device):
     """BASELINE config 2 (T=4096, E=128, k=4) and the routing of configs 4 / 5, plus a run with exact ties.  The small
     row counts run as one launch (top-k and metadata in one workgroup, at most two passes of its 1024 threads over the
-    rows: up to 256, 128, 64 or 32 rows for up to 64, 128, 256 or 512 experts); the cases sit on both sides of that."""
+    rows: up to 256, 128, 64 or 32 rows for up to 64, 128, 256 or 512 experts); beyond that two launches (top-k with a
+    histogram per workgroup, then ordering and tables) while there are at most 128 workgroups of rows that make whole
+    chunks of 64 entries (8192 rows of 128 logits; not k = 3 with 200 logits), else four.  The cases sit on both sides
+    of each limit."""
     torch.manual_seed(0)
     for ties in (False, True):
         logits = torch.randn(T, E)
@@ -147,3 +152,38 @@ def test_routing_configs(T, E, k, device):
         assert torch.equal(rm.block_schedule_data.cpu(), ref["ragged"].block_schedule_data)
         torch.testing.assert_close(out.vals.cpu(), ref["vals"], rtol=1e-5, atol=1e-6)
         assert int(out.col_sum.sum()) == T * k
+
+
+@pytest.mark.parametrize("T,E,k,dt", [(4096, 128, 4, torch.int16), (1500, 96, 4, torch.int32), (30000, 64, 4, torch.int32),
+                                      (40000, 64, 4, torch.int16), (700, 1000, 2, torch.int32), (6000, 1000, 2, torch.int32),
+                                      (64, 128, 4, torch.int16)])
+def test_routing_metadata_entry_point(T, E, k, dt, device):
+    """tamd_routing_metadata on given indices with dropped rows (-1) at the end, against the oracle: one launch for the
+    smallest case, two launches up to 128 blocks of 1024 entries, three beyond (40000 rows)."""
+    from oracle.routing_ref import bitmatrix_metadata_ref, ragged_metadata_ref
+    from triton_amd import _lib
+    from triton_amd.tensor_details.ragged_tensor import alloc_tables
+    torch.manual_seed(5)
+    indx = torch.rand(T, E).argsort(dim=1)[:, :k].to(dt)
+    indx[T - T // 8:] = -1
+    n = T * k
+    L = _lib.lib()
+    d = indx.to(device)
+    col_sum = torch.full((E, ), -7, dtype=torch.int32, device=device)
+    combined = torch.full((3 * n, ), -7, dtype=torch.int32, device=device)
+    offs, sched, width = alloc_tables(E, n, device)
+    ws = torch.empty(L.tamd_bitmatrix_metadata_workspace(n, E), dtype=torch.int32, device=device)
+    rc = L.tamd_routing_metadata(_lib.ptr(d), int(dt == torch.int16), n, E, k, _lib.ptr(col_sum), _lib.ptr(combined),
+                                 _lib.ptr(combined[n:]), _lib.ptr(combined[2 * n:]), _lib.ptr(offs), offs.stride(0),
+                                 _lib.ptr(sched), sched.stride(0), width, _lib.ptr(ws), _lib.stream_ptr(device))
+    assert rc == 0
+    ref = bitmatrix_metadata_ref(indx, E)
+    assert torch.equal(col_sum.cpu(), ref.col_sum)
+    assert torch.equal(combined[:n].cpu(), ref.col_sorted_indx)
+    assert torch.equal(combined[n:2 * n].cpu(), ref.row_sorted_indx)
+    gather = torch.div(ref.col_sorted_indx, k, rounding_mode="trunc")
+    assert torch.equal(combined[2 * n:].cpu(), gather)
+    rag = ragged_metadata_ref(ref.col_sum, n)
+    assert torch.equal(offs[0, :E + 1].cpu(), rag.slice_offs)
+    assert torch.equal(offs[1:, :E + 1].cpu(), rag.block_offs_data)
+    assert torch.equal(sched[:, :width].cpu(), rag.block_schedule_data)

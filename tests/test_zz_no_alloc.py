@@ -34,9 +34,10 @@ def _run(indx, E, k, static):
 
 def test_static_workspace_entry_point_matches_the_allocating_one(device):
     torch.manual_seed(11)
-    # (rows, experts, k): the first needs the three-launch path with ~150 KB of workspace, the second is smaller and
-    # still beyond the single-workgroup path, the third takes the single-workgroup path (no workspace at all)
-    for T, E, k, dt in ((4096, 128, 4, torch.int16), (1500, 96, 4, torch.int32), (64, 128, 4, torch.int16)):
+    # (rows, experts, k): the first needs the three-launch path with ~1.4 MB of workspace, the second and third the
+    # two-launch path, the fourth takes the single-workgroup path (no workspace at all)
+    for T, E, k, dt in ((40000, 128, 4, torch.int16), (4096, 128, 4, torch.int16), (1500, 96, 4, torch.int32),
+                        (64, 128, 4, torch.int16)):
         indx = torch.stack([torch.randperm(E)[:k] for _ in range(T)]).to(dt)
         indx[T - T // 8:] = -1  # dropped rows at the end
         indx = indx.to(device)

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(1024) void hist_kernel(const void *__restrict__ ind
     int run = 0;
     for (int c = 0; c < CH; ++c) {
       int t = hist[c * E + e];
-      chunk_pref[((int64_t)blk * CH + c) * E + e] = run;
+      if (chunk_pref) chunk_pref[((int64_t)blk * CH + c) * E + e] = run;  // (not needed by order_scan_kernel)
       run += t;
     }
     block_tot[(int64_t)blk * E + e] = run;
@@ -498,6 +498,202 @@ __global__ __launch_bounds__(1024) void scan_ragged_kernel(int E, int n_blocks, 
   const int64_t first = per * blockIdx.x;
   if (first < total_e)
     ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, first, per < total_e - first ? per : total_e - first);
+}
+
+// ---------------------------------------------------------------------------
+// metadata in two launches (up to kMaxTableBlocks blocks of chunks)
+// ---------------------------------------------------------------------------
+// The first launch leaves one histogram per block of CH chunks (hist_kernel, or topk_hist_kernel straight from the
+// logits).  In the second, every workgroup reduces that small table by itself -- the experts' totals, their prefix and,
+// for the workgroup that orders block `blk`, the counts of the blocks before it -- instead of waiting for a scan kernel
+// in between: workgroups 0..nb-1 recount their own chunks and place their entries, the remaining ones build the ragged
+// tables and fill the block schedule.
+constexpr int kMaxTableBlocks = 128;
+
+// Sums of tot[b][e] over the blocks b of [b_lo, b_hi): all of them, and those before block `blk`.  Sixteen loads are
+// in flight together.
+TAMD_DEVICE void sum_block_range(const int32_t *__restrict__ tot, int E, int e, int b_lo, int b_hi, int blk, int &all,
+                                 int &below) {
+  all = 0;
+  below = 0;
+  for (int b0 = b_lo; b0 < b_hi; b0 += 16) {
+    int t[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) t[u] = tot[(int64_t)(b0 + u < b_hi ? b0 + u : b_hi - 1) * E + e];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) asm volatile("" : "+v"(t[u]));
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      all += b0 + u < b_hi ? t[u] : 0;
+      below += b0 + u < b_hi && b0 + u < blk ? t[u] : 0;
+    }
+  }
+}
+
+__global__ __launch_bounds__(1024) void order_scan_kernel(const void *__restrict__ indx, int is16, int n, int E, int CH,
+                                                          int nbits, int k, const int32_t *__restrict__ block_tot, int nb,
+                                                          int P, int32_t *__restrict__ col_sum,
+                                                          int32_t *__restrict__ col_sorted, int32_t *__restrict__ row_sorted,
+                                                          int32_t *__restrict__ gather, int32_t *__restrict__ offs,
+                                                          int64_t offs_pitch, int32_t *__restrict__ sched,
+                                                          int64_t sched_pitch, int max_blocks) {
+  extern __shared__ int32_t sm[];
+  int32_t *hist = sm;                          // [CH][E]  counts of this block's chunks, then their exclusive prefix
+  int32_t *tot = hist + (int64_t)CH * E;       // [E]      entries per expert
+  int32_t *boff = tot + E;                     // [E]      entries per expert in the blocks before this one
+  int32_t *psum = boff + E;                    // [P][E]   partial sums over ranges of blocks
+  int32_t *pbel = psum + (int64_t)P * E;       // [P][E]
+  int32_t *tab = pbel + (int64_t)P * E;        // [6][E + 1]
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int blk = blockIdx.x;
+  const bool orders = blk < nb;
+  // this wave's chunk of the index array: requested first, used after the table has been reduced
+  const int i = (blk * CH + wave) * 64 + lane;
+  const bool has = orders && wave < CH && i < n;
+  int ev = 0;
+  if (n > 0) ev = load_indx(indx, is16, has ? i : 0);
+  if (orders)
+    for (int j = tid; j < CH * E; j += 1024) hist[j] = 0;
+  // 1. partial sums of the table: thread (part, e) takes the blocks [part * per, (part + 1) * per)
+  {
+    const int part = tid / E, e = tid - part * E;
+    if (part < P) {
+      const int per = (nb + P - 1) / P;
+      const int b_hi = (part + 1) * per < nb ? (part + 1) * per : nb;
+      int all, below;
+      sum_block_range(block_tot, E, e, part * per, b_hi, blk, all, below);
+      psum[part * E + e] = all;
+      pbel[part * E + e] = below;
+    }
+  }
+  asm volatile("" : "+v"(ev));
+  ev = has ? ev : -1;
+  __syncthreads();
+  // 2. totals per expert; counts of this wave's chunk
+  for (int e = tid; e < E; e += 1024) {
+    int all = 0, below = 0;
+    for (int q = 0; q < P; ++q) {
+      all += psum[q * E + e];
+      below += pbel[q * E + e];
+    }
+    tot[e] = all;
+    boff[e] = below;
+    if (blk == 0) col_sum[e] = all;
+  }
+  const bool valid = ev >= 0 && ev < E;
+  const uint64_t same = same_id_mask(ev, valid, nbits);
+  if (valid && (same & lanemask_lt()) == 0) hist[wave * E + ev] = __popcll(same);
+  __syncthreads();
+  // 3. exclusive prefix over this block's chunks; the ragged tables (row 0: exclusive prefix over the experts)
+  if (orders) {
+    for (int e = tid; e < E; e += 1024) {
+      int run = 0;
+      for (int c = 0; c < CH; ++c) {
+        const int v = hist[c * E + e];
+        hist[c * E + e] = run;
+        run += v;
+      }
+    }
+  }
+  ragged_scan_rows(tot, E, tab, blk == nb ? offs : nullptr, offs_pitch);
+  __syncthreads();
+  if (orders) {
+    // 4. placement
+    const int nv = tab[E];
+    if (valid) {
+      const int pos = tab[ev] + boff[ev] + hist[wave * E + ev] + __popcll(same & lanemask_lt());
+      row_sorted[i] = pos;
+      col_sorted[pos] = i;
+      if (gather) gather[pos] = i / k;
+    } else if (wave < CH && i < n) {
+      row_sorted[i] = -1;
+    }
+    if (wave < CH && i >= nv && i < n) {
+      col_sorted[i] = -1;
+      if (gather) gather[i] = 0;  // trunc(-1 / k)
+    }
+  } else {
+    // 4'. this workgroup's share of the block schedule
+    const int64_t total = 5 * (int64_t)max_blocks;
+    const int64_t shares = (int64_t)gridDim.x - nb;
+    const int64_t per = (total + shares - 1) / shares;
+    const int64_t first = per * (blk - nb);
+    if (first < total) ragged_fill_schedule(tab, E, sched, sched_pitch, max_blocks, first, per < total - first ? per : total - first);
+  }
+}
+
+// Second launch of the two: the grid, the LDS size and the limits of order_scan_kernel.
+inline bool order_scan_applicable(int64_t n, int E, int CH, int64_t nb) {
+  if (E > 1024 || nb < 1 || nb > kMaxTableBlocks || n > 0x7FFFFFFF - 64 * 1024) return false;
+  int P = 1024 / E;
+  P = P > 16 ? 16 : P;
+  const int64_t ints = (int64_t)CH * E + 2 * (int64_t)E + 2 * (int64_t)P * E + 6 * ((int64_t)E + 1);
+  return ints * 4 <= 150 * 1024;
+}
+
+inline int launch_order_scan(const void *indx, int is16, int64_t n, int E, int CH, int nbits, int k, const int32_t *block_tot,
+                             int64_t nb, int32_t *col_sum, int32_t *col_sorted, int32_t *row_sorted, int32_t *gather,
+                             int32_t *offs, int64_t offs_pitch, int32_t *sched, int64_t sched_pitch, int max_blocks,
+                             hipStream_t st) {
+  int P = 1024 / E;
+  P = P > 16 ? 16 : P;
+  P = P > nb ? (int)nb : P;
+  const int64_t ints = (int64_t)CH * E + 2 * (int64_t)E + 2 * (int64_t)P * E + 6 * ((int64_t)E + 1);
+  int64_t shares = (5 * (int64_t)max_blocks + 4095) / 4096;  // about four schedule entries per thread
+  shares = shares < 1 ? 1 : (shares > 64 ? 64 : shares);
+  if (int rc = raise_lds_limit_once((const void *)order_scan_kernel)) return rc;
+  order_scan_kernel<<<dim3((unsigned)(nb + shares)), 1024, (size_t)ints * 4, st>>>(
+      indx, is16, (int)n, E, CH, nbits, k, block_tot, (int)nb, P, col_sum, col_sorted, row_sorted, gather, offs, offs_pitch,
+      sched, sched_pitch, max_blocks);
+  return launch_status();
+}
+
+// First launch of the two, from the logits: the experts of 1024 / L rows per workgroup (their picked columns also go to
+// LDS) and the histogram of that block of (1024 / L) * k / 64 whole chunks.
+template <int DT, int L, int EPL>
+__global__ __launch_bounds__(1024) void topk_hist_kernel(const void *__restrict__ x, int64_t x_stride, int n_rows, int E,
+                                                         int k, void *__restrict__ y_vals, int16_t *__restrict__ y_indx,
+                                                         uint32_t *__restrict__ bits, int64_t bits_stride_row,
+                                                         int64_t bits_stride_word, int nbits, int CH,
+                                                         int32_t *__restrict__ block_tot) {
+  extern __shared__ int32_t sm[];
+  constexpr int ROWS = 1024 / L;
+  int32_t *lidx = sm;            // [CH * 64] picked columns of this block's rows
+  int32_t *hist = sm + CH * 64;  // [CH][E]
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+  for (int j = tid; j < CH * E; j += 1024) hist[j] = 0;  // (the barrier below covers them)
+  topk_row<DT, L, EPL>(x, x_stride, n_rows, E, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row, bits_stride_word,
+                       row0 + tid / L, lidx - row0 * k);
+  __syncthreads();
+  if (wave < CH) {
+    const int j = wave * 64 + lane;  // entry of the block; its row exists or not
+    const bool valid = row0 + j / k < n_rows;
+    const int e = valid ? lidx[j] : -1;
+    const uint64_t same = same_id_mask(e, valid, nbits);
+    if (valid && (same & lanemask_lt()) == 0) hist[wave * E + e] = __popcll(same);
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += 1024) {
+    int run = 0;
+    for (int c = 0; c < CH; ++c) run += hist[c * E + e];
+    block_tot[(int64_t)blockIdx.x * E + e] = run;
+  }
+}
+
+template <int DT>
+int launch_topk_hist(const void *x, int64_t xs, int n_rows, int E, int k, void *yv, int16_t *yi, uint32_t *bits, int64_t bsr,
+                     int64_t bsw, int nbits, int L, int CH, int32_t *block_tot, hipStream_t st) {
+  const size_t lds = ((size_t)CH * 64 + (size_t)CH * E) * 4;
+  const unsigned grid = (unsigned)((n_rows + 1024 / L - 1) / (1024 / L));
+#define TAMD_TH(LL, EE) \
+  topk_hist_kernel<DT, LL, EE><<<grid, 1024, lds, st>>>(x, xs, n_rows, E, k, yv, yi, bits, bsr, bsw, nbits, CH, block_tot)
+  if (L == 8) TAMD_TH(8, 8);
+  else if (L == 16) TAMD_TH(16, 8);
+  else if (L == 32) TAMD_TH(32, 8);
+  else TAMD_TH(64, 8);
+#undef TAMD_TH
+  return launch_status();
 }
 
 // ---------------------------------------------------------------------------
@@ -802,6 +998,18 @@ static int routing_metadata_impl(const void *indx, int indx_is_int16, int64_t n_
       return launch_status();
     }
   }
+  {
+    // two launches while the table of block histograms is small enough for every workgroup to reduce by itself
+    const MetaPlan p = make_meta_plan(n_indx, n_cols);
+    if (order_scan_applicable(n_indx, n_cols, p.CH, p.n_blocks)) {
+      hipStream_t st = (hipStream_t)stream;
+      hist_kernel<<<dim3((unsigned)p.n_blocks), 1024, (size_t)p.CH * n_cols * 4, st>>>(
+          indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, nullptr, workspace + p.off_block_tot);
+      return launch_order_scan(indx, indx_is_int16, n_indx, n_cols, p.CH, p.nbits, k, workspace + p.off_block_tot, p.n_blocks,
+                               col_sum, col_sorted_indx, row_sorted_indx, gather_indx, offs, offs_pitch, schedule, sched_pitch,
+                               max_n_blocks, st);
+    }
+  }
   const size_t sr_lds = ((size_t)n_cols + 6 * ((size_t)n_cols + 1) + 17) * 4;
   if (sr_lds <= 150 * 1024) {
     // three launches: histograms per workgroup, scans + ragged tables, placement
@@ -864,6 +1072,29 @@ extern "C" int tamd_routing(const void *logits, int dtype, int64_t stride, int n
       if (dtype == TAMD_BF16) TAMD_RFD(TAMD_BF16);
       TAMD_RFD(TAMD_F16);
 #undef TAMD_RFD
+    }
+    // two launches: top-k with the histogram of each workgroup's rows, then ordering and tables.  The rows of a
+    // workgroup (1024 / L) must make whole chunks of 64 entries.
+    const int CH = 16 * k / L;
+    const int64_t nb = ((int64_t)n_rows + 1024 / L - 1) / (1024 / L);
+    if ((16 * k) % L == 0 && CH >= 1 && CH <= 16 && workspace && order_scan_applicable(n, n_cols, CH, nb) &&
+        nb * n_cols <= tamd_bitmatrix_metadata_workspace(n, n_cols)) {
+      int nbits = 0;
+      while ((1 << nbits) < n_cols) ++nbits;
+      hipStream_t st = (hipStream_t)stream;
+      int rc;
+      if (dtype == TAMD_F32)
+        rc = launch_topk_hist<TAMD_F32>(logits, stride, n_rows, n_cols, k, y_vals, y_indx, bits, bits_stride_row,
+                                        bits_stride_word, nbits, L, CH, workspace, st);
+      else if (dtype == TAMD_BF16)
+        rc = launch_topk_hist<TAMD_BF16>(logits, stride, n_rows, n_cols, k, y_vals, y_indx, bits, bits_stride_row,
+                                         bits_stride_word, nbits, L, CH, workspace, st);
+      else
+        rc = launch_topk_hist<TAMD_F16>(logits, stride, n_rows, n_cols, k, y_vals, y_indx, bits, bits_stride_row,
+                                        bits_stride_word, nbits, L, CH, workspace, st);
+      if (rc != 0) return rc;
+      return launch_order_scan(y_indx, 1, n, n_cols, CH, nbits, k, workspace, nb, col_sum, col_sorted_indx, row_sorted_indx,
+                               gather_indx, offs, offs_pitch, schedule, sched_pitch, max_n_blocks, st);
     }
   }
   const int rc = tamd_topk_forward(logits, dtype, stride, n_rows, n_cols, k, 1, 0, y_vals, y_indx, k, bits, bits_stride_row,
