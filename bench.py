@@ -253,9 +253,9 @@ def run_routing(args, cfg, name):
     out = base_line(args, "moe_routing_tokens_per_s", round(T / (wall * 1e-3), 1), "tokens/s", wall, "f32 logits -> int32",
                     f"{name}: routing (top-{k} of {E} + softmax, histogram, gather / scatter indices, ragged tables), T={T}")
     out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "topk_kernel + 3 metadata kernels",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "topk_hist_kernel + order_scan_kernel",
                        "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes,
-                       "note": "2.4 MB in four launches: bound by launch latency, not by HBM"}
+                       "note": "2.4 MB in two launches: bound by launch latency, not by HBM"}
     out["cpu_baseline"] = {"value": round(T / cpu_s, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
                            "sample": f"oracle routing_ref (numpy) on the whole batch, {cpu_s:.3f} s"}
     out["parity"] = {"routing_bit_exact": ok, "softmax_values_within_1e-5": vals_ok}
