@@ -454,6 +454,29 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
     const int cpr = OUT_COLS / epc;           // chunks per tile row
     const int n_chunks = t.rows * cpr;
     if constexpr (PRE) {
+      // Usual case -- every chunk of the tile lies wholly inside or wholly outside the output's columns and lands on a
+      // 16-byte boundary: the staged chunks are read first, then each is stored under one predicate and no other
+      // control flow (the general loop below compiles to a state machine per chunk that takes several times longer).
+      constexpr int EPC_C = 16 / OSZ_C;
+      const bool whole_chunks =
+          n_out % EPC_C == 0 &&
+          ((((uintptr_t)a.y) | (uintptr_t)(a.y_stride_m * OSZ_C) | (uintptr_t)(a.y_stride_z * OSZ_C)) & 15) == 0;
+      if (whole_chunks) {
+        uint4 staged_chunk[MAXU];
+#pragma unroll
+        for (int u = 0; u < MAXU; ++u) staged_chunk[u] = *(const uint4 *)(ob + (size_t)(tid + u * 256) * 16);
+#pragma unroll
+        for (int u = 0; u < MAXU; ++u) {
+          const int id = tid + u * 256;
+          const int r = id / CPR_C, c = (id - r * CPR_C) * EPC_C;
+          const int gcol = tile_out0 + c;
+          if (id < n_chunks && dst_row[u] >= 0 && gcol < n_out) {
+            uint8_t *yp = (uint8_t *)a.y + ((int64_t)t.z * a.y_stride_z + (int64_t)dst_row[u] * a.y_stride_m + gcol) * OSZ_C;
+            *(uint4 *)yp = staged_chunk[u];
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int u = 0; u < MAXU; ++u) {
         const int id = tid + u * 256;
