@@ -187,3 +187,27 @@ def test_routing_metadata_entry_point(T, E, k, dt, device):
     assert torch.equal(offs[0, :E + 1].cpu(), rag.slice_offs)
     assert torch.equal(offs[1:, :E + 1].cpu(), rag.block_offs_data)
     assert torch.equal(sched[:, :width].cpu(), rag.block_schedule_data)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [100, 1000])
+def test_routing_16bit_logits(dtype, T, device):
+    """16-bit logits (many exact ties) through the one-launch and the two-launch routing: indices and every table
+    bit-exact, gate weights to the output type's rounding."""
+    torch.manual_seed(7)
+    E, k = 128, 4
+    logits = torch.randn(T, E).to(dtype)
+    out = routing(logits.to(device), k)
+    ref = R.routing_ref(logits, k)
+    assert torch.equal(out.indx.cpu().int(), ref["indx"])
+    assert torch.equal(out.col_sum.cpu(), ref["col_sum"])
+    assert torch.equal(out.scatter_indx.cpu(), ref["scatter_indx"])
+    assert torch.equal(out.row_sorted_indx.cpu(), ref["row_sorted_indx"])
+    assert torch.equal(out.gather_indx.cpu(), ref["gather_indx"])
+    rm = out.ragged_metadata
+    assert torch.equal(rm.block_offs_data.cpu(), ref["ragged"].block_offs_data)
+    assert torch.equal(rm.block_schedule_data.cpu(), ref["ragged"].block_schedule_data)
+    assert out.vals.dtype == dtype
+    torch.testing.assert_close(out.vals.cpu().float(), ref["vals"].float(), rtol=2e-2, atol=1e-3)
+    sp = out.sparse
+    assert torch.equal(sp.mask.storage.data.cpu().view(torch.int32), R.topk_ref(logits, k)[2])
