@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const void *__restrict__ x,
   const int64_t nv = (S1 + VEC - 1) / VEC;
   const int64_t total = S0 * nv;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const int64_t s0 = i / nv, c0 = (i - s0 * nv) * VEC;
+    const int64_t s0 = total <= 0x7FFFFFFF ? (int64_t)((uint32_t)i / (uint32_t)nv) : i / nv, c0 = (i - s0 * nv) * VEC;
     float acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
@@ -235,7 +235,8 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
   for (int64_t base = (int64_t)blockIdx.x * 256; base < total; base += (int64_t)gridDim.x * 256) {
     const int64_t i = base + threadIdx.x;
     const bool live = i < total;
-    const int64_t s0 = live ? i / threads_per_row : 0;
+    // (a 64-bit division costs about a hundred instructions per thread; the index usually fits 32 bits)
+    const int64_t s0 = !live ? 0 : (total <= 0x7FFFFFFF ? (int64_t)((uint32_t)i / (uint32_t)threads_per_row) : i / threads_per_row);
     const int64_t c0 = live ? (i - s0 * threads_per_row) * PV : S1;  // c0 >= S1: a padding thread of the row
     float acc[PV];
 #pragma unroll
@@ -303,11 +304,19 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
                   v[2 * j + 1] = a.x_dtype == TAMD_BF16 ? bf16_bits_to_f32(w[j] >> 16) : f16_bits_to_f32(w[j] >> 16);
                 }
               } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                  const int b = (int)(((j < 4 ? q[u][0].x : q[u][0].y) >> (8 * (j & 3))) & 0xFFu);
-                  v[j] = a.x_dtype == TAMD_FP8_E4M3 ? __builtin_amdgcn_cvt_f32_fp8(b, 0) : __builtin_amdgcn_cvt_f32_bf8(b, 0);
+                // two values per conversion instruction (the pair is picked by an immediate)
+                typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                const int w0 = (int)q[u][0].x, w1 = (int)q[u][0].y;
+                f32x2_t p[4];
+                if (a.x_dtype == TAMD_FP8_E4M3) {
+                  p[0] = __builtin_amdgcn_cvt_pk_f32_fp8(w0, false), p[1] = __builtin_amdgcn_cvt_pk_f32_fp8(w0, true);
+                  p[2] = __builtin_amdgcn_cvt_pk_f32_fp8(w1, false), p[3] = __builtin_amdgcn_cvt_pk_f32_fp8(w1, true);
+                } else {
+                  p[0] = __builtin_amdgcn_cvt_pk_f32_bf8(w0, false), p[1] = __builtin_amdgcn_cvt_pk_f32_bf8(w0, true);
+                  p[2] = __builtin_amdgcn_cvt_pk_f32_bf8(w1, false), p[3] = __builtin_amdgcn_cvt_pk_f32_bf8(w1, true);
                 }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[2 * j] = p[j][0], v[2 * j + 1] = p[j][1];
               }
 #pragma unroll
               for (int j = 0; j < PV; ++j) acc[j] += v[j % 8] * flex_in;
