@@ -201,3 +201,23 @@ def test_reduce_refuses_what_is_not_built(device):
         reduce(x, 1, unpadded_batch_size=torch.tensor([2], device=device))
     with pytest.raises(NotImplementedError):
         reduce(x, 1, y_value_pack_factor=2, y_has_mx=True)
+
+
+@pytest.mark.parametrize("shape,dim", [((512, 4, 2880), 1), ((3, 64, 4, 512), 2), ((5, 4, 100), 1), ((64, 7, 264), 1)])
+@pytest.mark.parametrize("x_dtype", [torch.float8_e4m3fn, torch.float8_e5m2, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("y_dtype", [None, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("scales", ["none", "flex", "flex+global"])
+def test_reduce_plain_sums_of_fp8_and_scaled_rows(shape, dim, x_dtype, y_dtype, scales, device):
+    """The top-k combine of fp8 rows (and plain sums with only the scalar input scales): dense aligned shapes take the
+    kernel variant that compiles nothing but the vector paths, (5, 4, 100) the general one; bit for bit against the
+    index-order float32 sum of the oracle."""
+    from triton_amd.numerics import InFlexData
+    torch.manual_seed(3)
+    x = torch.randn(shape).to(x_dtype)
+    fscale = torch.tensor([0.5]) if scales != "none" else None
+    gscale = torch.tensor([3.0]) if scales == "flex+global" else None
+    y, y_mx = reduce(x.to(device), dim=dim, x_flex=InFlexData(scale=fscale.to(device)) if fscale is not None else InFlexData(),
+                     x_global_scale=None if gscale is None else gscale.to(device), y_dtype=y_dtype)
+    ry, _, _ = MR.reduce_general_ref(x, dim, x_flex_scale=fscale, x_global_scale=gscale, y_dtype=y_dtype)
+    assert y_mx is None and y.dtype == (y_dtype or x_dtype) and tuple(y.shape) == tuple(ry.shape)
+    assert torch.equal(y.cpu().view(torch.uint8), ry.contiguous().view(torch.uint8))

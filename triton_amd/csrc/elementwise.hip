@@ -218,7 +218,11 @@ TAMD_DEVICE uint32_t narrow_bits(float v, int dt) {  // 8- or 16-bit output type
   return dt == TAMD_BF16 ? (f32_to_bf16_bits(v) & 0xFFFFu) : (dt == TAMD_F16 ? (f32_to_f16_bits(v) & 0xFFFFu) : f32_to_fp8_bits(v, dt));
 }
 
-template <int PV, int RN>
+// LEAN: plain sums of dense, aligned rows (no mask, no per-element or block scales, no pairwise post-processing, no
+// flexpoint or MXFP8 output; the scalar input scales may be there) -- what the top-k combine of fp8 rows is.  Only
+// the vector paths are compiled, which takes the kernel from 143 to about half as many registers: it is bound by
+// the loads it has in flight, i.e. by how many of its waves fit a CU.
+template <int PV, int RN, bool LEAN = false>
 __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int64_t threads_per_row, int vec_in, int vec_out) {
   constexpr int NO = PV / RN;                         // outputs per thread
   constexpr int TPG = 32 / NO > 0 ? 32 / NO : 1;      // threads of one 32-column output group
@@ -245,7 +249,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
       // PV values of row r of the reduced axis
       auto load_row = [&](int64_t r, float (&v)[PV]) {
         const int64_t xo = s0 * a.xs0 + r * a.xsr;
-        if (PV == 8 && vec_in) {  // unit inner stride, 8 columns inside S1, 8-element alignment of every row
+        if (LEAN || (PV == 8 && vec_in)) {  // unit inner stride, 8 columns inside S1, 8-element alignment of every row
           if (xsz == 4) {
             const float4 lo = *(const float4 *)((const float *)a.x + xo + c0), hi = *(const float4 *)((const float *)a.x + xo + c0 + 4);
             v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4 % PV] = hi.x, v[5 % PV] = hi.y, v[6 % PV] = hi.z, v[7 % PV] = hi.w;
@@ -271,7 +275,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
         }
       };
       int64_t r = 0;
-      if (PV == 8 && vec_in && !a.x_mx_scale && !a.scale && !a.mask) {
+      if (LEAN || (PV == 8 && vec_in && !a.x_mx_scale && !a.scale && !a.mask)) {
         // plain sums (the top-k combine): four rows are fetched together -- raw loads first, conversions after, with
         // the element size fixed outside so that no branch separates the loads -- and added in the order r = 0, 1, ...
         auto batches = [&](auto xs_tag) {
@@ -330,6 +334,11 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
       for (; r < a.R; ++r) {
         float v[PV];
         load_row(r, v);
+        if constexpr (LEAN) {
+#pragma unroll
+          for (int j = 0; j < PV; ++j) acc[j] += v[j] * flex_in;
+          continue;
+        }
 #pragma unroll
         for (int j = 0; j < PV; ++j) {
           const int64_t c = c0 + j;
@@ -355,7 +364,9 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
       o[j] *= global;
     }
     const int64_t oc0 = c0 / RN;  // first output column
-    if (a.y_mx_scale) {
+    if constexpr (LEAN) {
+      // nothing between the sums and the store
+    } else if (a.y_mx_scale) {
       // MXFP8: the group's threads are TPG neighbouring lanes (rows are padded to whole groups of threads)
       float m = 0.f;
 #pragma unroll
@@ -388,7 +399,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
     }
     if (oc0 >= Y_S1) continue;
     // ---- store: NO outputs, as one or two vector stores when the row is dense and aligned
-    if (NO > 1 && vec_out && oc0 + NO <= Y_S1) {
+    if (LEAN || (NO > 1 && vec_out && oc0 + NO <= Y_S1)) {
       uint8_t *yp = (uint8_t *)a.y + (s0 * a.ys0 + oc0) * ysz;
       if (ysz == 4) {
 #pragma unroll
@@ -424,7 +435,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
       }
     }
   }
-  if (a.y_actual_scale && !a.y_mx_scale) {
+  if (!LEAN && a.y_actual_scale && !a.y_mx_scale) {
     // wave maximum, then one atomic per wave; positive floats order like their bit patterns, NaN counts as +inf
 #pragma unroll
     for (int sh = 32; sh > 0; sh >>= 1) {
@@ -438,7 +449,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
   }
 }
 
-template <int PV, int RN>
+template <int PV, int RN, bool LEAN = false>
 int launch_reduce_ex(const tamd_reduce_args &a, int vec_in, int vec_out, hipStream_t st) {
   constexpr int NO = PV / RN;
   constexpr int TPG = 32 / NO > 0 ? 32 / NO : 1;
@@ -447,7 +458,7 @@ int launch_reduce_ex(const tamd_reduce_args &a, int vec_in, int vec_out, hipStre
   const int64_t total = a.S0 * tpr;
   int64_t blocks = (total + 255) / 256;
   blocks = blocks > 65536 * 16 ? 65536 * 16 : (blocks < 1 ? 1 : blocks);
-  reduce_ex_kernel<PV, RN><<<dim3((unsigned)blocks), 256, 0, st>>>(a, tpr, vec_in, vec_out);
+  reduce_ex_kernel<PV, RN, LEAN><<<dim3((unsigned)blocks), 256, 0, st>>>(a, tpr, vec_in, vec_out);
   return launch_status();
 }
 
@@ -538,6 +549,9 @@ extern "C" int tamd_reduce_ex(const tamd_reduce_args *args, void *stream) {
   const int no = 8 / rn;
   const int vec_out = wide && a.ys1 == 1 && (a.S1 / rn) % no == 0 && aligned(a.y, no * ysz < 16 ? no * ysz : 16) &&
                       (a.ys0 * ysz) % (no * ysz < 16 ? no * ysz : 16) == 0;
+  const bool lean = wide && rn == 1 && vec_in && vec_out && !a.mask && !a.scale && !a.x_mx_scale && !a.y_mx_scale &&
+                    !a.y_expected_scale && !a.y_actual_scale;
+  if (lean) return launch_reduce_ex<8, 1, true>(a, vec_in, vec_out, st);
   if (wide) return rn == 1 ? launch_reduce_ex<8, 1>(a, vec_in, vec_out, st) : launch_reduce_ex<8, 2>(a, vec_in, vec_out, st);
   return rn == 1 ? launch_reduce_ex<1, 1>(a, 0, 0, st) : launch_reduce_ex<2, 2>(a, 0, 0, st);
 }
