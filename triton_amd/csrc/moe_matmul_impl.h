@@ -726,6 +726,36 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, kb >> 1);
     }
   };
+  // Paired form (ring mode, row blocks of up to 64 rows): the weights of stages 2p and 2p + 1 are 128 contiguous bytes
+  // of every column and are requested as such -- eight lanes per column, so that a column's piece is one 128-byte
+  // request where it lies inside a line instead of two of 64 bytes a stage apart.  With few rows per expert these
+  // requests are what keeps each CU's address unit and L1 busy.  Instruction j copies positions 8j + lane/8 (128 bytes
+  // each, wave-private 8 KB); slot lane%8 of position p holds the column's 16-byte part (lane%8) ^ ((p>>1)&7), which
+  // keeps the operand reads of 16 consecutive positions on distinct banks.
+  constexpr bool PAIRED = RING && DA == 3;
+  const uint32_t lds_b2 = lds_base + DA * A_STAGE + wave * 8192;
+  const uint8_t *bbuf2 = lds + DA * A_STAGE + wave * 8192;
+  uint32_t w2_off[PAIRED ? 8 : 1];
+  int w2_part[PAIRED ? 8 : 1];
+  if constexpr (PAIRED) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int pos = j * 8 + lane / 8;
+      const int col = t.n0 + wave * 64 + 2 * (pos % 32) + pos / 32;
+      w2_part[j] = (lane % 8) ^ ((pos >> 1) & 7);
+      w2_off[j] = (uint32_t)(col < N ? col : N - 1) * (uint32_t)a.w_stride_n + w2_part[j] * 16;
+    }
+  }
+  auto issue_b_pair = [&](int pair) {
+    if constexpr (PAIRED) {
+      const int kb = pair * 256;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t bkill = (wave_live && kb + w2_part[j] * 32 < K) ? 0u : kOob;
+        dma16(rw, lds_b2 + j * 1024, w2_off[j] | bkill, kb >> 1);
+      }
+    }
+  };
   // ring mode: the scales of weight stage `sup` for this wave's 64 columns, into the wave's 1 KB piece of the scale
   // ring.  Pre-shuffled layout: one copy -- the wave's two blocks of 32 columns hold the 8 groups that contain the
   // stage's 4 as 256 contiguous bytes each (lanes 0-15 / 16-31; the other lanes copy nothing).  Strided layout:
@@ -760,18 +790,23 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
   };
 
-  uint4 raw[NF][2];
+  // (two register sets: the ring loop for row blocks of up to 64 rows keeps the weights of two stages)
+  uint4 raw[2][NF][2];
   float scf[NF][2];      // 16-bit path: 2^(e-127) as a float
-  uint32_t scw[NF];      // fp8 path: scale bytes of q = 0, 1 in bytes 0, 1
-  // registers <- this wave's weights and scales of super-stage `sup`
-  auto load_b = [&](int sup) {
+  uint32_t scw[2][NF];   // fp8 path: scale bytes of q = 0, 1 in bytes 0, 1
+  // registers (set `set`) <- this wave's weights and scales of super-stage `sup`
+  auto load_b = [&](int sup, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
 #pragma unroll
     for (int f = 0; f < NF; ++f)
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int pos = f * 32 + c32;
-        raw[f][q] = *(const uint4 *)(bbuf + (DB == 2 ? (sup & 1) * B_BYTES : 0) + pos * 64 +
-                                     (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
+        if constexpr (PAIRED)
+          raw[set][f][q] = *(const uint4 *)(bbuf2 + pos * 128 + (((4 * (sup & 1) + 2 * q + h) ^ ((pos >> 1) & 7)) * 16));
+        else
+          raw[set][f][q] = *(const uint4 *)(bbuf + (DB == 2 ? (sup & 1) * B_BYTES : 0) + pos * 64 +
+                                            (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
         // group kg = 4*sup + 2q + h of this lane's column.  Strided: byte kg, kept inside the column's G bytes
         // (groups past the end of K meet zero codes and zero activations; their scale only has to be some finite
         // value of this column).  Pre-shuffled: byte 256*(kg/8) + 64*(kg%4) + 2*((kg%8)/4); the padding up to a
@@ -788,7 +823,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         } else if constexpr (SC_LDS) sbyte = lds_sc[sc_col_off[f] + kg_off];
         else if (cdna4) sbyte = s_base[sc_col_off[f] + kg_off];
         else sbyte = s_base[(int64_t)(col0 + f < N ? col0 + f : N - 1) * a.w_mx_stride_n + kg_off];
-        if constexpr (FP8) scw[f] = q == 0 ? sbyte : (scw[f] | (sbyte << 8));
+        if constexpr (FP8) scw[set][f] = q == 0 ? sbyte : (scw[set][f] | (sbyte << 8));
         else scf[f][q] = bits_to_f32(sbyte << 23);
       }
   };
@@ -822,8 +857,9 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
   };
 
-  auto compute = [&](int it, auto qc) {
+  auto compute = [&](int it, auto qc, auto set_c) {
     constexpr int q = decltype(qc)::value;
+    constexpr int set = decltype(set_c)::value;
     if (!wave_live) return;
     const uint8_t *buf = lds + a_slot(it) * A_STAGE;
     if constexpr (FP8) {
@@ -835,16 +871,16 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         if (s == 0) fp8_read_frags(buf, 1, af8[1]);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
-          const uint4 r = raw[f][s];
+          const uint4 r = raw[set][f][s];
           const i32x8_t bf = i32x8_t{(int)r.x, (int)r.y, (int)r.z, (int)r.w, 0, 0, 0, 0};
 #pragma unroll
           for (int i = 0; i < NFR; ++i) {
             if (s == 0)
               acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[0][i], bf, acc[i][f], CBSZ, 4, 0, sa8[i], 0,
-                                                                        (int)scw[f]);
+                                                                        (int)scw[set][f]);
             else
               acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[1][i], bf, acc[i][f], CBSZ, 4, 2, sa8[i], 1,
-                                                                        (int)scw[f]);
+                                                                        (int)scw[set][f]);
           }
         }
       }
@@ -861,7 +897,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         if (s < 3) read_frags(s + 1, af[(s + 1) & 1]);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
-          const uint4 r = raw[f][q];
+          const uint4 r = raw[set][f][q];
           const uint32_t codes = s == 0 ? r.x : (s == 1 ? r.y : (s == 2 ? r.z : r.w));
           const frag_t bf = M::expand(codes, scf[f][q]);
 #pragma unroll
@@ -871,36 +907,61 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
   };
 
+  typedef std::integral_constant<int, 0> Set0;
+  typedef std::integral_constant<int, 1> Set1;
   if constexpr (RING) {
-    // Stage s requests the activations of stage s + DA - 1 and then the weights and scales of stage s + 2 (the weight
-    // buffer of stage s is free as soon as its contents are in registers).  Copies complete in the order of their
-    // requests, so what may still be in flight at the top of a stage is: with three activation stages, everything the
-    // stage before requested; with two, only the weights and scales it requested (5 copies, or 8 with strided scales).
+    // Copies complete in the order of their requests, so a stage waits by count for what it needs and leaves the
+    // later requests in flight.
     const bool as_wave = x_mx && wave * 64 < LDS_ROWS;
     constexpr int NSC = 4;  // scale copies of a stage with strided scales (1 when pre-shuffled)
-    if constexpr (DA == 3) {
-      issue_a(0), issue_as(0), issue_b(0), issue_sc(0);
-      issue_a(1), issue_as(1), issue_b(1), issue_sc(1);
+    if constexpr (PAIRED) {
+      // Three activation stages; an even stage s moves the weights of s and s + 1 into registers and requests those of
+      // s + 2 and s + 3 (one pair), the odd stage requests only activations.
+      issue_a(0), issue_as(0);
+      issue_b_pair(0), issue_sc(0), issue_sc(1);
+      issue_a(1), issue_as(1);
+      for (int it = 0; it < n_ka; it += 2) {
+        // in flight at most: the activations of stage it + 1
+        if (as_wave) wait_vmcnt<NFR + 4>(); else wait_vmcnt<NFR>();
+        __syncthreads();
+        load_b(it, Set0{});
+        load_b(it + 1, Set1{});
+        fp8_read0(it);
+        issue_a(it + 2);
+        issue_as(it + 2);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: their buffer may be refilled
+        issue_b_pair((it >> 1) + 1);
+        issue_sc(it + 2), issue_sc(it + 3);
+        compute(it, Set0{}, Set0{});
+        if (it + 1 < n_ka) {
+          // in flight at most: everything the even stage requested
+          if (cdna4) { if (as_wave) wait_vmcnt<NFR + 4 + 8 + 2>(); else wait_vmcnt<NFR + 8 + 2>(); }
+          else { if (as_wave) wait_vmcnt<NFR + 4 + 8 + 2 * NSC>(); else wait_vmcnt<NFR + 8 + 2 * NSC>(); }
+          __syncthreads();
+          fp8_read0(it + 1);
+          issue_a(it + 3);
+          issue_as(it + 3);
+          compute(it + 1, Set0{}, Set1{});
+        }
+      }
     } else {
+      // Stage s requests the activations of stage s + 1 and then the weights and scales of stage s + 2 (the weight
+      // buffer of stage s is free as soon as its contents are in registers): in flight at the top of a stage are at
+      // most the weights and scales the stage before requested (5 copies, or 8 with strided scales).
       issue_b(0), issue_sc(0);
       issue_a(0), issue_as(0), issue_b(1), issue_sc(1);
-    }
-    for (int it = 0; it < n_ka; ++it) {
-      if constexpr (DA == 3) {
-        if (cdna4) { if (as_wave) wait_vmcnt<NFR + 4 + 4 + 1>(); else wait_vmcnt<NFR + 4 + 1>(); }
-        else { if (as_wave) wait_vmcnt<NFR + 4 + 4 + NSC>(); else wait_vmcnt<NFR + 4 + NSC>(); }
-      } else {
+      for (int it = 0; it < n_ka; ++it) {
         if (cdna4) wait_vmcnt<4 + 1>(); else wait_vmcnt<4 + NSC>();
+        __syncthreads();
+        load_b(it, Set0{});
+        fp8_read0(it);
+        issue_a(it + DA - 1);
+        issue_as(it + DA - 1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: their buffer may be refilled
+        issue_b(it + 2);
+        issue_sc(it + 2);
+        compute(it, Set0{}, Set0{});
       }
-      __syncthreads();
-      load_b(it);
-      fp8_read0(it);
-      issue_a(it + DA - 1);
-      issue_as(it + DA - 1);
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: their buffer may be refilled
-      issue_b(it + 2);
-      issue_sc(it + 2);
-      compute(it, std::integral_constant<int, 0>{});
     }
   } else {
   issue_a(0);
@@ -910,30 +971,30 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     for (int it = 0; it < n_ka; ++it) {  // activation and weight stages coincide (128 K each)
       wait_dma();
       __syncthreads();
-      load_b(it);
+      load_b(it, Set0{});
       fp8_read0(it);
       issue_a(it + 1);
       issue_as(it + 1);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
       issue_b(it + 1);
-      compute(it, std::integral_constant<int, 0>{});
+      compute(it, Set0{}, Set0{});
     }
   } else {
     for (int it = 0; it < n_ka; it += 2) {
       wait_dma();
       __syncthreads();
-      load_b(it >> 1);
+      load_b(it >> 1, Set0{});
       issue_a(it + 1);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
       issue_b((it >> 1) + 1);
-      compute(it, std::integral_constant<int, 0>{});
+      compute(it, Set0{}, Set0{});
       if (it + 1 < n_ka) {
         // the weight copies just issued (4, after the activation stage it + 1) are not needed before the next
         // even stage and take the longest (weights stream from HBM, activations mostly hit L2): leave them in flight
         wait_vmcnt<4>();
         __syncthreads();
         issue_a(it + 2);
-        compute(it + 1, std::integral_constant<int, 1>{});
+        compute(it + 1, Set1{}, Set0{});
       }
     }
   }
