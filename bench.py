@@ -111,11 +111,17 @@ def spin_up(fn):
         torch.cuda.synchronize()
 
 
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
 def timed(fn, steps, warmup):
     """Runs fn warmup + steps times for the wall time per call, then steps times again with a pair of HIP events around
     every call for the kernel time: for calls of a few tens of microseconds the event records themselves (host time and
     marker packets between the kernels) would otherwise be a third of the step they are meant to measure.  Returns
-    (results of the last call, mean HIP-event ms around a call, wall ms per call of the uninstrumented pass)."""
+    (results of the last call, median HIP-event ms around a call, wall ms per call of the uninstrumented pass)."""
     out = None
     spin_up(fn)
     for _ in range(warmup):
@@ -134,7 +140,7 @@ def timed(fn, steps, warmup):
     torch.cuda.synchronize()
     # back to back, the wall time per call bounds the time of the call's kernels from above: where the events (which add
     # a marker packet on either side) read more than that, the bound is the better figure
-    return out, min(sum(a.elapsed_time(b) for a, b in ev) / steps, wall), wall
+    return out, min(median([a.elapsed_time(b) for a, b in ev]), wall), wall
 
 
 def base_line(args, metric, value, unit, ms_per_step, dtype, workload_text, **config):
@@ -401,8 +407,8 @@ def run_fc2(args, cfg, name):
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    kernel_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    combine_ms = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
+    kernel_ms = median([e[0].elapsed_time(e[1]) for e in events])
+    combine_ms = median([e[2].elapsed_time(e[3]) for e in events])
     flops = 2.0 * rows * K * N
     col_sum = r.col_sum.cpu()
     n_active = int((col_sum > 0).sum())
@@ -422,6 +428,14 @@ def run_fc2(args, cfg, name):
                     algorithmic_flops=flops, frac_of_mxfp4_peak=round(tflops_kernel / PEAK_MXFP4_TFLOPS, 4),
                     hbm_gbs=round(gbs_kernel, 1))
     combine_bytes = rows * N * 2 + T * N * 2
+    # the least a fused matmul + combine would move (rows, weights, gate weights and scatter indices in, the combined
+    # tokens out); what ran is the reference's two-kernel form, whose intermediate rows are written and read once more
+    fused_min = rows * K + n_active * (K // 2 * N + K // 32 * N + N * 2) + rows * 8 + T * N * 2
+    roof["form"] = "two kernels: matmul_ogs writes bf16 [rows, N] (scattered), reduce sums the k slots"
+    roof["algorithmic_bytes_fused_minimum"] = fused_min
+    roof["algorithmic_bytes_two_kernel_form"] = mm_bytes + combine_bytes
+    if traffic is not None:
+        roof["traffic_over_fused_minimum"] = round(traffic / fused_min, 3)
     roof["combine"] = dict(kernel="reduce_kernel", kernel_ms=round(combine_ms, 4), bound="hbm", algorithmic_bytes=combine_bytes,
                            achieved=round(combine_bytes / (combine_ms * 1e-3) / 1e9, 1), unit="GB/s",
                            frac=round(combine_bytes / (combine_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4))
@@ -507,7 +521,7 @@ def run_fc1(args, cfg, name):
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    kernel_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    kernel_ms = median([a.elapsed_time(b) for a, b in events])
 
     col_sum = r.col_sum.cpu()
     rows = T * k
@@ -633,7 +647,7 @@ def run_mlp(args, cfg, name):
         logits, r, y1, y2, z = step(events[i])
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    stage_ms = {n: sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i, n in enumerate(names)}
+    stage_ms = {n: median([e[i].elapsed_time(e[i + 1]) for e in events]) for i, n in enumerate(names)}
     rows = T * k
     flops = {"gate_matmul": 2.0 * T * d1 * E, "fc1_swiglu": 2.0 * rows * d1 * d2, "fc2_scatter": 2.0 * rows * (d2 // 2) * d1}
     n_active = int((r.col_sum > 0).sum())
@@ -665,7 +679,11 @@ def run_mlp(args, cfg, name):
     # fp8 outputs: one step of the type (2^-3 relative) where an fp32 sum lands on a rounding boundary
     fc1_ok = bool(torch.allclose(y1[:n_rows].cpu().float(), y1_ref.float(), rtol=0.13, atol=2e-2))
     got2 = y2.cpu()[ref["scatter_indx"][:n_rows].long()].float()
-    fc2_ok = bool(torch.allclose(torch.nan_to_num(got2, nan=1e30), torch.nan_to_num(y2_ref.float(), nan=1e30), rtol=0.13, atol=1.0))
+    # NaN marks an overflowed float8_e4m3fn output: the pattern of NaNs must agree, everything else within one step
+    ref2 = y2_ref.float()
+    nan_frac = float(torch.isnan(ref2).float().mean())
+    fc2_ok = bool(torch.equal(torch.isnan(got2), torch.isnan(ref2)) and
+                  torch.allclose(torch.nan_to_num(got2, nan=0.0), torch.nan_to_num(ref2, nan=0.0), rtol=0.13, atol=2e-2))
     z_ref, _, _ = MR.reduce_general_ref(y2.view(T, k, d1)[:256].cpu(), 1)
     a, b = z[:256].cpu().float(), z_ref.float()
     combine_ok = bool(torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a), torch.nan_to_num(b)))
@@ -686,7 +704,8 @@ def run_mlp(args, cfg, name):
                            "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
                            "sample": f"oracle FC1 + FC2 on the first {n_e} of {E} experts ({n_rows} of {rows} rows), {cpu_s:.1f} s"}
     out["parity"] = {"gate_logits_within_2e-2": logits_ok, "routing_bit_exact": routing_ok, "fc1_sample_within_fp8_step": fc1_ok,
-                     "fc2_sample_within_fp8_step": fc2_ok, "combine_bit_exact": combine_ok}
+                     "fc2_sample_within_fp8_step": fc2_ok, "fc2_sample_overflowed_fraction": round(nan_frac, 5),
+                     "combine_bit_exact": combine_ok}
     return out
 
 
@@ -734,12 +753,11 @@ def main():
     ap.add_argument("--block-m", type=int, default=0)
     ap.add_argument("--scale-layout", default=None, choices=["strided", "cdna4"],
                     help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
-                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout())).  Default: strided, except for "
-                    "--workload mlp, which hands over the pre-shuffled scales as the reference's bench_mlp does on this "
-                    "target (make_default_matmul_mxfp4_w_scale_layout, tensor_details/layout.py:43-54)")
+                    "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout())).  Default: cdna4, what the reference "
+                    "picks on this target (make_default_matmul_mxfp4_w_scale_layout, tensor_details/layout.py:43-54)")
     args = ap.parse_args()
     if args.scale_layout is None:
-        args.scale_layout = "cdna4" if args.workload == "mlp" else "strided"
+        args.scale_layout = "cdna4"
     args.cpu_work = 1.0
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported (with more GPUs the experts "

@@ -165,8 +165,14 @@ int tamd_routing(const void *logits, int dtype, int64_t stride, int n_rows, int 
  * (tamd_bitmatrix_metadata_workspace(n_indx, n_cols) int32 elements) exceeds
  * tamd_routing_metadata_static_max_workspace() elements return TAMD_E_TOO_LARGE and launch nothing.  All calls on
  * one GPU share that array: calls that overlap in time on the same GPU (different streams or threads) race; calls
- * on one stream are ordered and safe.
+ * on one stream are ordered and safe.  Nothing in the array has to start at zero (every entry a launch reads is
+ * written earlier by the same call).
+ * One-time host-side set-up per device (the array's address by hipGetSymbolAddress, the raised dynamic-LDS limits of
+ * three kernels by hipFuncSetAttribute) happens on a device's first call, or ahead of time in
+ * tamd_routing_metadata_static_init() with that device current: a caller that records a graph calls init, or makes
+ * one ordinary call, before the capture begins.
  */
+int tamd_routing_metadata_static_init(void);
 int64_t tamd_routing_metadata_static_max_workspace(void);
 int tamd_routing_metadata_static(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
                                  int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
@@ -281,7 +287,9 @@ int tamd_reduce(const void *x, int x_dtype, int64_t S0, int64_t R, int64_t S1, i
  * (reduce.py:375-492 kernel body, :818-957 host, API :1135-1157).  x [S0, R, S1] -> y [S0, S1 / n] where n = 1
  * without post-processing and 2 with one of the pairwise functions below.
  *
- *   acc[s0, c] = sum_r mask * (x * 2^(x_mx_scale - 127) * *x_flex_scale * scale)       float32, r in index order
+ *   acc[s0, c] = sum_r mask * (x * 2^(x_mx_scale - 127) * *x_flex_scale * scale)       float32, r in index order; the
+ *                first term starts the sum when R <= 8 (reduce.py:137, 467-470: a column of -0.0 stays -0.0), longer
+ *                axes start from +0.0; a term with a scale is fma(x, scale, +0.0) (reduce.py:466)
  *   o          = postprocess(acc) * *x_global_scale
  *   flexpoint output (no y_mx_scale): *y_actual_scale <- max(*y_actual_scale, max|o| / max_finite(y_dtype) + 1e-30)
  *                                     by atomic max; o / *y_expected_scale, clamped to y_dtype's finite range when
@@ -319,6 +327,9 @@ typedef struct tamd_reduce_args {
   int y_saturate_inf;
   uint8_t *y_mx_scale; /* [S0, ceil(S1 / n / 32)] */
   int64_t yms0, yms1;
+  /* optional device scalar (reduce.py:550-555 of the reference, `unpadded_batch_size`): only rows s0 < *it are
+   * reduced and written; the rest of y (and of y_mx_scale) is left as it is */
+  const int32_t *unpadded_batch_size;
 } tamd_reduce_args;
 
 int tamd_reduce_ex(const tamd_reduce_args *args, void *stream);

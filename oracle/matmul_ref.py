@@ -135,13 +135,32 @@ def reduce_mx_ref(x: torch.Tensor, x_mxscale: torch.Tensor, dim: int, mask=None,
     return downcast_to_mxfp_ref(acc, torch.float8_e4m3fn, axis=-1)
 
 
+def _index_order_sum(xf: torch.Tensor, dim: int) -> torch.Tensor:
+    """float32 sum over `dim` in index order, one addition per step, started as the reference's kernel starts it
+    (reduce.py:137 `use_static_loop = K <= 8`, :423-424, :467-470): for an axis of at most 8 entries the first term IS
+    the initial value (so a column of -0.0 stays -0.0), longer axes start from +0.0."""
+    n = xf.shape[dim]
+    out_shape = [m for i, m in enumerate(xf.shape) if i != dim]
+    if n == 0:
+        return torch.zeros(out_shape, dtype=torch.float32)
+    if n <= 8:
+        acc = xf.select(dim, 0).clone()
+        first = 1
+    else:
+        acc = torch.zeros(out_shape, dtype=torch.float32)
+        first = 0
+    for r in range(first, n):
+        acc = acc + xf.select(dim, r)
+    return acc
+
+
 _MAX_FINITE = {torch.float8_e4m3fn: 448.0, torch.float8_e5m2: 57344.0, torch.float16: 65504.0,
                torch.bfloat16: 3.3895313892515355e38, torch.float32: 3.4028234663852886e38}
 
 
 def reduce_general_ref(x: torch.Tensor, dim: int, mask=None, scale=None, x_mxscale=None, x_flex_scale=None,
                        x_global_scale=None, postprocess=None, y_dtype=None, y_expected_scale=None,
-                       y_saturate_inf: bool = False, y_has_mx: bool = False):
+                       y_saturate_inf: bool = False, y_has_mx: bool = False, unpadded_batch_size=None):
     """reduce_torch (reduce.py:1179-1210 of the reference) together with the operands only its kernel has
     (_reduce_forward_inner, reduce.py:441-492): the order of the factors of a term ((x * 2^e) * x_flex_scale) * scale,
     x_global_scale after the post-processing function, the flexpoint output as float_to_flex computes it
@@ -149,20 +168,25 @@ def reduce_general_ref(x: torch.Tensor, dim: int, mask=None, scale=None, x_mxsca
     saturating).  Built from pieces that are pinned on their own -- upcast_from_mxfp_ref, swiglu_ref,
     downcast_to_mxfp_ref, torch's casts -- around an explicit index-order float32 sum.
 
-    postprocess: None, ("swiglu", alpha, limit) or ("plus_a", a).  Returns (y, y_mxscale or None, actual_scale)."""
+    postprocess: None, ("swiglu", alpha, limit) or ("plus_a", a).  unpadded_batch_size: only that many entries of the
+    first kept axis are reduced (reduce.py:550-555, 694-695; the kernel leaves the other rows of y alone), and only
+    they are returned.  Returns (y, y_mxscale or None, actual_scale)."""
     from .mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
     y_dtype = y_dtype or x.dtype
+    if unpadded_batch_size is not None:
+        d0 = [d for d in range(x.ndim) if d != dim % x.ndim][0]
+        n = int(unpadded_batch_size)
+        narrow = lambda t: None if t is None else (t.narrow(d0, 0, n) if t.shape[d0] != 1 else t)
+        x, mask, scale, x_mxscale = narrow(x), narrow(mask), narrow(scale), narrow(x_mxscale)
     xf = upcast_from_mxfp_ref(x, x_mxscale, torch.float32, axis=-1) if x_mxscale is not None else x.to(torch.float32)
     if x_flex_scale is not None:
         xf = xf * x_flex_scale.to(torch.float32)
     if scale is not None:
-        xf = xf * scale.to(torch.float32)
+        xf = xf * scale.to(torch.float32) + torch.zeros((), dtype=torch.float32)  # tl.fma(x, s, 0.0), reduce.py:466
     if mask is not None:
         xf = torch.where(mask.to(torch.bool), xf, torch.zeros((), dtype=torch.float32))
     dim = dim % xf.ndim
-    acc = torch.zeros([n for i, n in enumerate(xf.shape) if i != dim], dtype=torch.float32)
-    for r in range(xf.shape[dim]):
-        acc = acc + xf.select(dim, r)
+    acc = _index_order_sum(xf, dim)
     if postprocess is not None:
         if postprocess[0] == "swiglu":
             acc = swiglu_ref(acc, postprocess[1], postprocess[2])

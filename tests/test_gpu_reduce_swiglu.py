@@ -198,8 +198,6 @@ def test_reduce_refuses_what_is_not_built(device):
     with pytest.raises(NotImplementedError):
         reduce(x, 1, postprocess_fn1=PostprocessFn(FnSpecs("gelu", None, (), reduction_n=1), ()))
     with pytest.raises(NotImplementedError):
-        reduce(x, 1, unpadded_batch_size=torch.tensor([2], device=device))
-    with pytest.raises(NotImplementedError):
         reduce(x, 1, y_value_pack_factor=2, y_has_mx=True)
 
 
@@ -221,3 +219,52 @@ def test_reduce_plain_sums_of_fp8_and_scaled_rows(shape, dim, x_dtype, y_dtype, 
     ry, _, _ = MR.reduce_general_ref(x, dim, x_flex_scale=fscale, x_global_scale=gscale, y_dtype=y_dtype)
     assert y_mx is None and y.dtype == (y_dtype or x_dtype) and tuple(y.shape) == tuple(ry.shape)
     assert torch.equal(y.cpu().view(torch.uint8), ry.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn])
+@pytest.mark.parametrize("with_mask", [True, False])
+def test_reduce_unpadded_batch_size(dtype, with_mask, device):
+    """tests/test_reduce.py:156-176 of the reference: B, M, N = 7, 73, 257 reduced over B with a device-side count of 37
+    rows; the rows past it keep what y held."""
+    torch.manual_seed(0)
+    B, M, N, unpadded, sentinel = 7, 73, 257, 37, -1234.0
+    x = torch.randn(B, M, N).to(dtype)
+    y_dtype = torch.float16 if dtype == torch.float8_e4m3fn else dtype
+    mask = torch.ones((B, M, 1), dtype=torch.int8).expand(B, M, N) if with_mask else None
+    y = torch.full((M, N), sentinel, dtype=y_dtype, device=device)
+    got, _ = reduce(x.to(device), dim=0, mask=None if mask is None else mask.to(device), y=y, y_dtype=y_dtype,
+                    unpadded_batch_size=torch.tensor(unpadded, device=device, dtype=torch.int32))
+    want, _, _ = MR.reduce_general_ref(x, 0, y_dtype=y_dtype, unpadded_batch_size=torch.tensor(unpadded))
+    assert got.data_ptr() == y.data_ptr()
+    assert torch.equal(got[:unpadded].cpu().view(torch.uint8), want.contiguous().view(torch.uint8))
+    assert torch.equal(got[unpadded:].cpu(), torch.full((M - unpadded, N), sentinel, dtype=y_dtype))
+    # a count beyond the axis reduces every row; zero reduces none
+    y2 = torch.full((M, N), sentinel, dtype=y_dtype, device=device)
+    reduce(x.to(device), dim=0, y=y2, y_dtype=y_dtype, unpadded_batch_size=torch.tensor(10 ** 6, device=device, dtype=torch.int32))
+    full, _, _ = MR.reduce_general_ref(x, 0, y_dtype=y_dtype)
+    assert torch.equal(y2.cpu().view(torch.uint8), full.contiguous().view(torch.uint8))
+    y3 = torch.full((M, N), sentinel, dtype=y_dtype, device=device)
+    reduce(x.to(device), dim=0, y=y3, y_dtype=y_dtype, unpadded_batch_size=torch.tensor(0, device=device, dtype=torch.int32))
+    assert torch.equal(y3.cpu(), torch.full((M, N), sentinel, dtype=y_dtype))
+
+
+@pytest.mark.parametrize("R", [1, 4, 8, 9])
+@pytest.mark.parametrize("shape_tail", [(2880, ), (33, )])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float8_e4m3fn])
+def test_reduce_sign_of_zero_follows_the_reference_kernel(R, shape_tail, dtype, device):
+    """Columns of -0.0: the first term starts the sum for an axis of at most 8 entries (reduce.py:137, 467-470 of the
+    reference), so the result is -0.0; a longer axis starts from +0.0.  With a scale every term passes through
+    fma(x, s, +0.0) and the result is +0.0; a masked first entry counts as +0.0."""
+    x = torch.full((16, R, *shape_tail), -0.0).to(dtype)
+    y_dtype = torch.bfloat16 if dtype == torch.float8_e4m3fn else dtype
+    y, _ = reduce(x.to(device), 1, y_dtype=y_dtype)
+    assert torch.signbit(y.float()).all().item() == (R <= 8)
+    want, _, _ = MR.reduce_general_ref(x, 1, y_dtype=y_dtype)
+    assert torch.equal(y.cpu().view(torch.uint8), want.contiguous().view(torch.uint8))
+    ys, _ = reduce(x.to(device), 1, scale=torch.ones((1, R, 1), device=device), y_dtype=y_dtype)
+    assert not torch.signbit(ys.float()).any().item()
+    mask = torch.ones((16, R, 1), dtype=torch.bool)
+    mask[::2, 0] = False
+    ym, _ = reduce(x.to(device), 1, mask=mask.to(device), y_dtype=y_dtype)
+    wm, _, _ = MR.reduce_general_ref(x, 1, mask=mask, y_dtype=y_dtype)
+    assert torch.equal(ym.cpu().view(torch.uint8), wm.contiguous().view(torch.uint8))

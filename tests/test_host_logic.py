@@ -179,3 +179,23 @@ x.h:9:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resourc
 """
     assert _scratch_users(remarks) == [("_ZN4tamd1aEv", 704)]
     assert _scratch_users("") == []
+
+
+def test_turned_gate_weights_are_cached_per_tensor_and_version():
+    """Weights with unit stride along N are turned once for the narrow-output kernel: the copy is reused while the
+    caller's tensor is alive and unmodified, redone after an in-place write, dropped with the tensor."""
+    import gc
+    import torch
+    from triton_amd import matmul as mm
+    w = torch.randn(64, 16)
+    t1 = mm._k_contiguous_cached(w)
+    assert t1.stride() == (1, 64) and torch.equal(t1, w)
+    assert mm._k_contiguous_cached(w) is t1
+    w.mul_(2.0)
+    t2 = mm._k_contiguous_cached(w)
+    assert t2 is not t1 and torch.equal(t2, w)
+    key = id(w)
+    assert key in mm._TURNED
+    del w
+    gc.collect()
+    assert key not in mm._TURNED

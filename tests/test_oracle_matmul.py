@@ -220,3 +220,30 @@ def test_reduce_general_ref_reduces_to_the_pinned_pieces():
     want = (x8.float() * 2.0)[:, 0] + (x8.float() * 2.0)[:, 1] + (x8.float() * 2.0)[:, 2]
     assert torch.equal(y, want)
     assert abs(float(actual) - (float(want.abs().max()) / 3.4028234663852886e38 + 1e-30)) < 1e-36
+
+
+def test_reduce_general_ref_sign_of_zero_and_unpadded_rows():
+    """What IEEE arithmetic makes of the reference kernel's start of the sum (reduce.py:137, 423-424, 466-470), worked by
+    hand: up to 8 entries the first term is the initial value, so -0.0 survives; a longer axis starts from +0.0 and
+    -0.0 + ... + -0.0 added to +0.0 is +0.0; a scale goes through fma(x, s, +0.0), and (-0.0 * s) + 0.0 is +0.0; a
+    masked first entry is loaded as +0.0, and +0.0 + -0.0 is +0.0."""
+    neg = lambda t: torch.signbit(t).tolist()
+    one = torch.full((1, 1, 2), -0.0)
+    y, _, _ = MR.reduce_general_ref(one, 1)
+    assert neg(y) == [[True, True]]
+    four = torch.full((1, 4, 2), -0.0)
+    y, _, _ = MR.reduce_general_ref(four, 1)
+    assert neg(y) == [[True, True]]
+    nine = torch.full((1, 9, 2), -0.0)
+    y, _, _ = MR.reduce_general_ref(nine, 1)
+    assert neg(y) == [[False, False]]
+    y, _, _ = MR.reduce_general_ref(four, 1, scale=torch.ones(1, 4, 1))
+    assert neg(y) == [[False, False]]
+    mask = torch.tensor([[[0, 1], [1, 1], [1, 1], [1, 1]]], dtype=torch.bool)
+    y, _, _ = MR.reduce_general_ref(four, 1, mask=mask)
+    assert neg(y) == [[False, True]]
+    # only the first `unpadded_batch_size` entries of the first kept axis are reduced (tests/test_reduce.py:156-176 of the
+    # reference: y_ref = x[:, :unpadded, :].sum(0))
+    x = torch.arange(2 * 5 * 3, dtype=torch.float32).reshape(2, 5, 3)
+    y, _, _ = MR.reduce_general_ref(x, 0, unpadded_batch_size=torch.tensor(3))
+    assert torch.equal(y, x[0, :3] + x[1, :3])

@@ -10,6 +10,14 @@ from triton_amd.tensor_details.ragged_tensor import alloc_tables
 pytestmark = pytest.mark.gpu
 
 
+def _poison_static_workspace(device):
+    """Fills the static array with garbage through an ordinary call on other data, so that a following call cannot rely
+    on anything in it being zero (or being its own earlier output)."""
+    E, k, T = 128, 4, 40000
+    junk = torch.randint(0, E, (T, k), dtype=torch.int16, device=device)
+    _run(junk, E, k, static=True)
+
+
 def _run(indx, E, k, static):
     dev = indx.device
     n = indx.numel()
@@ -34,6 +42,7 @@ def _run(indx, E, k, static):
 
 def test_static_workspace_entry_point_matches_the_allocating_one(device):
     torch.manual_seed(11)
+    assert _lib.lib().tamd_routing_metadata_static_init() == 0
     # (rows, experts, k): the first needs the three-launch path with ~1.4 MB of workspace, the second and third the
     # two-launch path, the fourth takes the single-workgroup path (no workspace at all)
     for T, E, k, dt in ((40000, 128, 4, torch.int16), (4096, 128, 4, torch.int16), (1500, 96, 4, torch.int32),
@@ -42,9 +51,45 @@ def test_static_workspace_entry_point_matches_the_allocating_one(device):
         indx[T - T // 8:] = -1  # dropped rows at the end
         indx = indx.to(device)
         want = _run(indx, E, k, static=False)
+        _poison_static_workspace(device)
         got = _run(indx, E, k, static=True)
         for name, a, b in zip(("col_sum", "index arrays", "offsets", "schedule"), got, want):
             assert torch.equal(a, b), f"{name} differ for T={T}, E={E}"
+
+
+def test_static_entry_point_allocates_no_device_memory(device):
+    """Device memory in use (the driver's count and torch's) is the same before and after calls of the entry point
+    once the per-device set-up has run."""
+    L = _lib.lib()
+    assert L.tamd_routing_metadata_static_init() == 0
+    torch.manual_seed(5)
+    E, k = 128, 4
+    cases = []
+    for T in (4096, 40000, 64):
+        indx = torch.stack([torch.randperm(E)[:k] for _ in range(T)]).to(torch.int16).to(device)
+        n = indx.numel()
+        col_sum = torch.empty((E, ), dtype=torch.int32, device=device)
+        combined = torch.empty((3 * n, ), dtype=torch.int32, device=device)
+        offs, sched, width = alloc_tables(E, n, device)
+        cases.append((indx, n, col_sum, combined, offs, sched, width))
+    def call(indx, n, col_sum, combined, offs, sched, width):
+        return L.tamd_routing_metadata_static(_lib.ptr(indx), 1, n, E, k, _lib.ptr(col_sum), _lib.ptr(combined),
+                                              _lib.ptr(combined[n:]), _lib.ptr(combined[2 * n:]), _lib.ptr(offs),
+                                              offs.stride(0), _lib.ptr(sched), sched.stride(0), width,
+                                              _lib.stream_ptr(device))
+
+    for case in cases:  # every kernel the three paths launch has run once (the runtime loads code objects lazily)
+        assert call(*case) == 0
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(device)
+    torch0, reserved0 = torch.cuda.memory_allocated(device), torch.cuda.memory_reserved(device)
+    for case in cases:
+        rc = call(*case)
+        assert rc == 0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(device)
+    assert torch.cuda.memory_allocated(device) == torch0 and torch.cuda.memory_reserved(device) == reserved0
+    assert free1 == free0, f"device memory in use changed by {free0 - free1} bytes"
 
 
 def test_static_workspace_capacity_is_enforced(device):

@@ -94,6 +94,7 @@ class ReduceArgs(C.Structure):
         ("y", C.c_void_p), ("y_dtype", C.c_int), ("ys0", C.c_int64), ("ys1", C.c_int64),
         ("y_expected_scale", C.c_void_p), ("y_actual_scale", C.c_void_p), ("y_saturate_inf", C.c_int),
         ("y_mx_scale", C.c_void_p), ("yms0", C.c_int64), ("yms1", C.c_int64),
+        ("unpadded_batch_size", C.c_void_p),
     ]
 
 
@@ -114,6 +115,7 @@ _SIGNATURES = {
     "tamd_ragged_metadata": ([_PTR, _INT, _PTR, _I64, _PTR, _I64, _INT, _PTR], C.c_int),
     "tamd_routing_metadata": ([_PTR, _INT, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _I64, _INT,
                                _PTR, _PTR], C.c_int),
+    "tamd_routing_metadata_static_init": ([], C.c_int),
     "tamd_routing_metadata_static_max_workspace": ([], C.c_int64),
     "tamd_routing_metadata_static": ([_PTR, _INT, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _I64,
                                       _INT, _PTR], C.c_int),

@@ -81,9 +81,12 @@ __global__ __launch_bounds__(256) void reduce_kernel(const void *__restrict__ x,
   const int64_t total = S0 * nv;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t s0 = total <= 0x7FFFFFFF ? (int64_t)((uint32_t)i / (uint32_t)nv) : i / nv, c0 = (i - s0 * nv) * VEC;
+    // the first term starts the sum when the axis has at most 8 entries (reduce.py:137, 467-470 of the reference: a
+    // column of -0.0 stays -0.0), which is what a start from -0.0 does; longer axes start from +0.0
+    const float acc0 = (R > 0 && R <= 8) ? -0.0f : 0.0f;
     float acc[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+    for (int j = 0; j < VEC; ++j) acc[j] = acc0;
     int64_t r = 0;
     if constexpr (VEC == 8) {
       // plain sums (no mask, no scale: the top-k combine) fetch four rows at a time so that their loads overlap;
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(const void *__restrict__ x,
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         float t = v[j];
-        if (scale) t *= scale[s0 * ss0 + r * ssr + (c0 + j) * ss1];
+        if (scale) t = __builtin_fmaf(t, scale[s0 * ss0 + r * ssr + (c0 + j) * ss1], 0.0f);  // reduce.py:466
         if (mask && !mask[s0 * ms0 + r * msr + (c0 + j) * ms1]) t = 0.f;
         acc[j] += t;
       }
@@ -227,7 +230,13 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
   constexpr int NO = PV / RN;                         // outputs per thread
   constexpr int TPG = 32 / NO > 0 ? 32 / NO : 1;      // threads of one 32-column output group
   const int64_t S1 = a.S1, Y_S1 = S1 / RN;
-  const int64_t total = a.S0 * threads_per_row;
+  // rows past the device-side count are neither reduced nor written (reduce.py:550-555)
+  int64_t rows = a.S0;
+  if (a.unpadded_batch_size) {
+    const int64_t u = *a.unpadded_batch_size;
+    rows = u < 0 ? 0 : (u < rows ? u : rows);
+  }
+  const int64_t total = rows * threads_per_row;
   const int xsz = a.x_dtype == TAMD_F32 ? 4 : (is_fp8_type(a.x_dtype) ? 1 : 2);
   const int ysz = a.y_dtype == TAMD_F32 ? 4 : (is_fp8_type(a.y_dtype) ? 1 : 2);
   const float flex_in = a.x_flex_scale ? *a.x_flex_scale : 1.0f;
@@ -242,9 +251,12 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
     // (a 64-bit division costs about a hundred instructions per thread; the index usually fits 32 bits)
     const int64_t s0 = !live ? 0 : (total <= 0x7FFFFFFF ? (int64_t)((uint32_t)i / (uint32_t)threads_per_row) : i / threads_per_row);
     const int64_t c0 = live ? (i - s0 * threads_per_row) * PV : S1;  // c0 >= S1: a padding thread of the row
+    // the first term starts the sum when the axis has at most 8 entries (reduce.py:137, 467-470: a column of -0.0
+    // stays -0.0), which is what a start from -0.0 does; longer axes start from +0.0
+    const float acc0 = (a.R > 0 && a.R <= 8) ? -0.0f : 0.0f;
     float acc[PV];
 #pragma unroll
-    for (int j = 0; j < PV; ++j) acc[j] = 0.f;
+    for (int j = 0; j < PV; ++j) acc[j] = acc0;
     if (c0 < S1) {
       // PV values of row r of the reduced axis
       auto load_row = [&](int64_t r, float (&v)[PV]) {
@@ -348,7 +360,7 @@ __global__ __launch_bounds__(256) void reduce_ex_kernel(tamd_reduce_args a, int6
             t *= bits_to_f32(e << 23);
           }
           t *= flex_in;
-          if (a.scale && c < S1) t *= a.scale[s0 * a.ss0 + r * a.ssr + c * a.ss1];
+          if (a.scale && c < S1) t = __builtin_fmaf(t, a.scale[s0 * a.ss0 + r * a.ssr + c * a.ss1], 0.0f);  // reduce.py:466
           if (a.mask && c < S1 && !a.mask[s0 * a.ms0 + r * a.msr + c * a.ms1]) t = 0.f;
           acc[j] += c < S1 ? t : 0.f;
         }
@@ -550,7 +562,7 @@ extern "C" int tamd_reduce_ex(const tamd_reduce_args *args, void *stream) {
   const int vec_out = wide && a.ys1 == 1 && (a.S1 / rn) % no == 0 && aligned(a.y, no * ysz < 16 ? no * ysz : 16) &&
                       (a.ys0 * ysz) % (no * ysz < 16 ? no * ysz : 16) == 0;
   const bool lean = wide && rn == 1 && vec_in && vec_out && !a.mask && !a.scale && !a.x_mx_scale && !a.y_mx_scale &&
-                    !a.y_expected_scale && !a.y_actual_scale;
+                    !a.y_expected_scale && !a.y_actual_scale && !a.unpadded_batch_size;
   if (lean) return launch_reduce_ex<8, 1, true>(a, vec_in, vec_out, st);
   if (wide) return rn == 1 ? launch_reduce_ex<8, 1>(a, vec_in, vec_out, st) : launch_reduce_ex<8, 2>(a, vec_in, vec_out, st);
   return rn == 1 ? launch_reduce_ex<1, 1>(a, 0, 0, st) : launch_reduce_ex<2, 2>(a, 0, 0, st);

@@ -1127,6 +1127,18 @@ static int static_workspace(int32_t **out) {
 
 extern "C" int64_t tamd_routing_metadata_static_max_workspace(void) { return kStaticWorkspaceInts; }
 
+// Everything tamd_routing_metadata_static does once per device on the host side -- the address of the static array
+// and the raised LDS limits of the kernels the metadata path launches -- so that callers under graph capture can have
+// it done beforehand.  (tamd_routing_metadata_static does the same by itself on a device's first call.)
+extern "C" int tamd_routing_metadata_static_init(void) {
+  int32_t *ws = nullptr;
+  if (int rc = static_workspace(&ws)) return rc;
+  if (int rc = raise_lds_limit_once((const void *)meta_fused_kernel)) return rc;
+  if (int rc = raise_lds_limit_once((const void *)order_scan_kernel)) return rc;
+  if (int rc = raise_lds_limit_once((const void *)scan_ragged_kernel)) return rc;
+  return 0;
+}
+
 extern "C" int tamd_routing_metadata_static(const void *indx, int indx_is_int16, int64_t n_indx, int n_cols, int k,
                                             int32_t *col_sum, int32_t *col_sorted_indx, int32_t *row_sorted_indx,
                                             int32_t *gather_indx, int32_t *offs, int64_t offs_pitch,

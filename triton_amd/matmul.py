@@ -4,6 +4,7 @@ gfx950 kernels.  Argument names, defaults and error behaviour follow the
 reference; combinations that are not built raise NotImplementedError."""
 import ctypes
 import math
+import weakref
 from dataclasses import dataclass
 from typing import Callable, Optional
 
@@ -78,6 +79,21 @@ _DEFAULT_EPILOGUE = Epilogue(FnSpecs.default(), tuple(), tuple(), False)
 
 def _data(t):
     return t.storage.data if isinstance(t, Tensor) else t
+
+
+_TURNED = {}  # id(weights) -> (weak reference to them, their version counter, the copy with unit stride along K)
+
+
+def _k_contiguous_cached(w):
+    key = id(w)
+    hit = _TURNED.get(key)
+    if hit is not None and hit[0]() is w and hit[1] == w._version:
+        return hit[2]
+    turned = w.transpose(-1, -2).contiguous().transpose(-1, -2)
+    if len(_TURNED) >= 64:
+        _TURNED.clear()
+    _TURNED[key] = (weakref.ref(w, lambda _, key=key: _TURNED.pop(key, None)), w._version, turned)
+    return turned
 
 
 def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
@@ -199,8 +215,10 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if not b_fp4 and w.ndim == 2 and w.shape[-1] <= 128 and w.stride(-2) != 1 and w.shape[-2] % 8 == 0 \
             and a_ragged_metadata is None and gather_indx is None and scatter_indx is None:
         # a narrow dense product (the gate matmul: hidden -> expert logits): the kernel for it reads both operands
-        # along K, so weights stored with unit stride along N are turned once (a few hundred KB)
-        w = w.transpose(-1, -2).contiguous().transpose(-1, -2)
+        # along K, so weights stored with unit stride along N are turned (a few hundred KB); the turned copy is kept
+        # for as long as the caller's tensor lives and is not written to, so a layer that holds N-contiguous gate
+        # weights pays for the copy once
+        w = _k_contiguous_cached(w)
     _lib.require_gpu(a, "a")
     _lib.require_gpu(w, "b")
     assert a.stride(-1) == 1 or a.shape[-1] == 1, "a must be contiguous along K"

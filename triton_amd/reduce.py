@@ -77,7 +77,12 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
     index order; then the output's flexpoint scales or its MXFP8 quantisation along the last axis (when the input is
     microscaled, as in the reference, reduce.py:1185-1206); cast to y_dtype (default x.dtype)."""
     if unpadded_batch_size is not None:
-        raise NotImplementedError("unpadded_batch_size (a device-side row count) is not built")
+        # a device-side count of the rows of the first kept axis that hold data (reduce.py:694-695, 550-555): the rest
+        # of y is left as it is.  Read by the kernel, never on the host.
+        assert unpadded_batch_size.numel() == 1, "unpadded_batch_size is a single-element tensor"
+        _lib.require_gpu(unpadded_batch_size, "unpadded_batch_size")
+        if unpadded_batch_size.dtype != torch.int32:
+            unpadded_batch_size = unpadded_batch_size.to(torch.int32)
     if postprocess_fn2 is not None and postprocess_fn2.specs.name != "dflt":
         raise NotImplementedError("a second post-processing function is not built")
     if y_value_pack_factor != 1 or y_microblock_size != MXFP_BLOCK_SIZE:
@@ -100,6 +105,8 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
     if y_has_mx and y_actual is not None:
         raise NotImplementedError("a microscaled output keeps no flexpoint actual scale (reduce.py:480-484)")
     R = x.shape[dim]
+    if unpadded_batch_size is not None and x.ndim != 3:
+        raise NotImplementedError("unpadded_batch_size is built for 3-D inputs (the rows of the first kept axis)")
     if x.ndim == 3:
         # the reference's view (reduce.py:732-747): the two axes that stay are (S0, S1) with the strides they have
         d0, d1 = [d for d in range(3) if d != dim]
@@ -150,11 +157,13 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
             raise NotImplementedError("microscaled outputs are built as float8_e4m3fn values with e8m0 (uint8) scales")
     y_dtype = y_dtype or x.dtype
     plain = (x_mxscale is None and x_flex_scale is None and x_global_scale is None and pp == _lib.PP_NONE and not y_has_mx
-             and y_expected is None and y_actual is None and x.dtype.itemsize > 1 and y_dtype.itemsize > 1)
+             and y_expected is None and y_actual is None and x.dtype.itemsize > 1 and y_dtype.itemsize > 1
+             and unpadded_batch_size is None)
     if plain and mask is None and scale is None and y is None and R >= 512 and lead * tail <= (1 << 18) and x.is_contiguous():
         # a long axis over few outputs: a thread of the kernel walks the whole axis, so it is cut into chunks that
         # are summed side by side (float32 partial sums), then the chunks are summed
-        chunks = next((c for c in (64, 32, 16, 8) if R % c == 0), 0)
+        # (more than 8 chunks: the second sum then starts from +0.0 like the one long sum it stands for)
+        chunks = next((c for c in (64, 32, 16) if R % c == 0), 0)
         if chunks:
             lead_c = 1
             for n in x.shape[:dim]:
@@ -203,6 +212,7 @@ def reduce(x: torch.Tensor, dim: int, mask: Optional[torch.Tensor] = None, scale
     a.y_expected_scale = None if y_expected is None else y_expected.data_ptr()
     a.y_actual_scale = None if y_actual is None else y_actual.data_ptr()
     a.y_saturate_inf = int(bool(y_flex_saturate_inf))
+    a.unpadded_batch_size = None if unpadded_batch_size is None else unpadded_batch_size.data_ptr()
     y_mx = None
     if y_has_mx:
         y_mx = torch.empty([*out_shape[:-1], -(-out_shape[-1] // MXFP_BLOCK_SIZE)], dtype=torch.uint8, device=x.device)

@@ -107,9 +107,10 @@ def torch_dtype_to_dtype(dtype):
     raise AssertionError(f"Unknown dtype: {dtype}")
 
 
-def wrap_torch_tensor(t: torch.Tensor, dtype=None, shape=None, shape_max=None, layout=None) -> Tensor:
+def wrap_torch_tensor(torch_tensor: torch.Tensor, dtype=None, shape=None, shape_max=None, layout=None) -> Tensor:
     """Wraps a torch tensor.  For FP4 the logical shape doubles the unit-stride axis
     (two codes per byte); the layout records which axis that is."""
+    t = torch_tensor
     dtype = torch_dtype_to_dtype(t.dtype if dtype is None else dtype)
     strides = list(t.stride())
     if shape is None:
@@ -124,13 +125,19 @@ def wrap_torch_tensor(t: torch.Tensor, dtype=None, shape=None, shape_max=None, l
     return Tensor(Storage(t, layout), dtype=dtype, shape=shape, shape_max=shape_max)
 
 
-def empty(shape, dtype, device, layout=None) -> Tensor:
-    """Uninitialised tensor whose storage is contiguous along layout.major_dim."""
-    layout = layout if isinstance(layout, StridedLayout) else StridedLayout()
+def empty(shape, dtype, device, layout=None, allow_implicit_conversion: bool = False) -> Tensor:
+    """Uninitialised tensor whose storage is contiguous along layout.major_dim (reference tensor.py:300-317).  A
+    layout that is not strided is only accepted with `allow_implicit_conversion`: the tensor is then allocated in
+    the default strided layout and converted."""
+    initial = layout if isinstance(layout, StridedLayout) else StridedLayout()
     is_fp4 = dtype == FP4
-    sshape = layout.storage_shape(list(shape), is_fp4)
-    data = torch.empty_strided(sshape, layout.strides(sshape), dtype=dtype_to_torch_dtype(dtype), device=device)
-    return Tensor(Storage(data, layout), dtype=dtype, shape=list(shape))
+    sshape = initial.storage_shape(list(shape), is_fp4)
+    data = torch.empty_strided(sshape, initial.strides(sshape), dtype=dtype_to_torch_dtype(dtype), device=device)
+    ret = Tensor(Storage(data, initial), dtype=dtype, shape=list(shape))
+    assert layout is None or initial == layout or allow_implicit_conversion
+    if allow_implicit_conversion and layout is not None and initial != layout:
+        ret = convert_layout(ret, layout)
+    return ret
 
 
 def convert_layout(tensor: Tensor, layout: Layout) -> Tensor:
