@@ -191,6 +191,16 @@ def scales_for_matmul(scales, layout):
     return convert_layout(wrap_torch_tensor(scales), CDNA4MXScaleLayout())
 
 
+def weights_for_matmul(vals, layout):
+    """The weight codes in the encoding asked for on the command line: as downcast_to_mxfp leaves them (K contiguous per
+    column), or in the block layout of the gfx950 kernels (convert_layout(..., CDNA4MXValueLayout()))."""
+    if layout == "strided":
+        return vals
+    from triton_amd.tensor import FP4, convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import CDNA4MXValueLayout
+    return convert_layout(wrap_torch_tensor(vals, dtype=FP4), CDNA4MXValueLayout())
+
+
 def run_dense(args, cfg, name):
     """BASELINE config 1: y = x . deq(W) + bias, x bf16 [M, K], W fp32 [K, N] quantised to MXFP4 along K; the codes and
     scales of that quantisation are checked against the oracle bit for bit on the way."""
@@ -209,7 +219,8 @@ def run_dense(args, cfg, name):
     codes_ok = bool(torch.equal(vals.cpu(), rv) and torch.equal(scales.cpu(), rs))
     x, bias = x_cpu.to(dev), bias_cpu.to(dev)
     pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
-    y, kernel_ms, wall = timed(lambda: matmul(x, vals, bias, precision_config=pc), args.steps, args.warmup)
+    wq = weights_for_matmul(vals, args.value_layout)
+    y, kernel_ms, wall = timed(lambda: matmul(x, wq, bias, precision_config=pc), args.steps, args.warmup)
     flops = 2.0 * M * K * N
     alg_bytes = M * K * 2 + K // 2 * N + K // 32 * N + N * 2 + M * N * 2
     torch.set_num_threads(os.cpu_count())
@@ -220,7 +231,8 @@ def run_dense(args, cfg, name):
     gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
     out = base_line(args, "moe_matmul_ogs_tflops", round(flops / (wall * 1e-3) / 1e12, 2), "TFLOP/s", wall,
                     "bf16 x mxfp4 (fp32 accumulate)",
-                    f"{name}: dense matmul + bias, M={M}, K={K}, N={N}, W mxfp4 [{K},{N}]", scale_layout=args.scale_layout)
+                    f"{name}: dense matmul + bias, M={M}, K={K}, N={N}, W mxfp4 [{K},{N}]", scale_layout=args.scale_layout,
+                    value_layout=args.value_layout)
     out["matmul_kernel_tflops"] = round(flops / (kernel_ms * 1e-3) / 1e12, 2)
     out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                        "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_stream16_kernel",
@@ -379,13 +391,14 @@ def run_fc2(args, cfg, name):
                          flex_ctx=FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale)))
     y_buf = torch.empty((rows, N), dtype=torch.bfloat16, device=dev)
     constraints = {"block_m": args.block_m} if args.block_m else {}
+    wq = weights_for_matmul(vals, args.value_layout)
 
     def step(ev=None):
         r = routing(logits, k)
         gam = r.expert_sorted_gate_weights
         if ev is not None:
             ev[0].record()
-        y = matmul(x8, vals, bias, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam, c=y_buf)
+        y = matmul(x8, wq, bias, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam, c=y_buf)
         if ev is not None:
             ev[1].record()
             ev[2].record()
@@ -461,7 +474,7 @@ def run_fc2(args, cfg, name):
                     "fp8e4m3 x mxfp4 (fp32 accumulate)",
                     f"{name}: routing + matmul_ogs(fp8 rows, grouped GEMM, bias, gate weights, scatter) + "
                     f"top-{k} combine, T={T}, hidden={K}, experts={E}, W2 mxfp4 [{E},{K},{N}]",
-                    rows=rows, active_experts=n_active, scale_layout=args.scale_layout)
+                    rows=rows, active_experts=n_active, scale_layout=args.scale_layout, value_layout=args.value_layout)
     out.update({"tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
                 "roofline": roof, "cpu_baseline": cpu,
                 "parity": {"routing_bit_exact": routing_ok, "combine_bit_exact": combine_ok,
@@ -488,6 +501,7 @@ def run_fc1(args, cfg, name):
     pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
     fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if act else None
     constraints = {"block_m": args.block_m} if args.block_m else {}
+    wq = weights_for_matmul(vals, args.value_layout)
 
     mx8 = bool(cfg.get("mx8"))
     if mx8:
@@ -501,9 +515,9 @@ def run_fc1(args, cfg, name):
         if ev is not None:
             ev[0].record()
         if mx8:
-            y = matmul(xq, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pcs, fused_activation=fa)
+            y = matmul(xq, wq, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pcs, fused_activation=fa)
         else:
-            y = matmul(x, vals, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=fa)
+            y = matmul(x, wq, bias, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=fa)
         if ev is not None:
             ev[1].record()
         return r, y
@@ -575,7 +589,8 @@ def run_fc1(args, cfg, name):
                     ("mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") + " (fp32 accumulate)",
                     f"{name}: routing + " + ("downcast_to_mxfp(x) + " if mx8 else "") +
                     f"matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, hidden={K}, experts={E}, top-{k}, "
-                    f"W1 mxfp4 [{E},{K},{N}]", rows=rows, active_experts=n_active, scale_layout=args.scale_layout)
+                    f"W1 mxfp4 [{E},{K},{N}]", rows=rows, active_experts=n_active, scale_layout=args.scale_layout,
+                    value_layout=args.value_layout)
     out.update({"tokens_per_s": round(T / (ms_per_step * 1e-3), 1), "matmul_kernel_tflops": round(tflops_kernel, 2),
                 "roofline": roof, "cpu_baseline": cpu,
                 "parity": {"routing_bit_exact": routing_ok, "gemm_sample_within_1e-2": gemm_ok}})
@@ -617,6 +632,7 @@ def run_mlp(args, cfg, name):
     w2, s2 = quantise(d2 // 2, d1)
     x8 = rnd(T, d1).to(torch.float8_e4m3fn)
     x16 = x8.to(torch.bfloat16)
+    w1q, w2q = weights_for_matmul(w1, args.value_layout), weights_for_matmul(w2, args.value_layout)
     pc1 = PrecisionConfig(b_mx_scale=scales_for_matmul(s1, args.scale_layout), b_microblock_size=32)
     pc2 = PrecisionConfig(b_mx_scale=scales_for_matmul(s2, args.scale_layout), b_microblock_size=32)
     act1 = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.0, 1.0))
@@ -629,9 +645,9 @@ def run_mlp(args, cfg, name):
         mark(1)
         r = routing(logits, k)
         mark(2)
-        y1 = matmul(x8, w1, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
+        y1 = matmul(x8, w1q, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
         mark(3)
-        y2 = matmul(y1, w2, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
+        y2 = matmul(y1, w2q, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
         mark(4)
         z, _ = reduce(y2.view(T, k, d1), dim=1)
         mark(5)
@@ -693,7 +709,8 @@ def run_mlp(args, cfg, name):
     out = base_line(args, "moe_mlp_tokens_per_s", round(T / (ms_per_step * 1e-3), 1), "tokens/s", ms_per_step,
                     "fp8e4m3 x mxfp4 (fp32 accumulate), bf16 gate",
                     f"{name}: gate matmul + routing + FC1/SwiGLU + FC2 + combine, tokens={T}, d_model={d1}, experts={E}, "
-                    f"top-{k}, W1 mxfp4 [{E},{d1},{d2}], W2 mxfp4 [{E},{d2 // 2},{d1}]", scale_layout=args.scale_layout)
+                    f"top-{k}, W1 mxfp4 [{E},{d1},{d2}], W2 mxfp4 [{E},{d2 // 2},{d1}]", scale_layout=args.scale_layout,
+                    value_layout=args.value_layout)
     out["stages"] = stages
     out["roofline"] = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                        "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": None, "kernel": "mm_x8_mxfp4_kernel (FC1 + FC2)",
@@ -755,6 +772,10 @@ def main():
                     help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
                     "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout())).  Default: cdna4, what the reference "
                     "picks on this target (make_default_matmul_mxfp4_w_scale_layout, tensor_details/layout.py:43-54)")
+    ap.add_argument("--value-layout", default="blocks", choices=["strided", "blocks"],
+                    help="encoding of the MXFP4 weight codes handed to matmul: K contiguous per column, as "
+                    "downcast_to_mxfp leaves them and the reference's AMD path keeps them (tensor_details/layout.py:27-40), or "
+                    "the block layout of the gfx950 kernels (convert_layout(..., CDNA4MXValueLayout()); default)")
     args = ap.parse_args()
     if args.scale_layout is None:
         args.scale_layout = "cdna4"

@@ -45,6 +45,9 @@ extern "C" {
 /* encodings of the weight scales (tamd_matmul_args.w_mx_layout) */
 #define TAMD_SCALE_STRIDED 0
 #define TAMD_SCALE_CDNA4 1
+/* encodings of MXFP4 weight codes (tamd_matmul_args.w_layout) */
+#define TAMD_W_STRIDED 0
+#define TAMD_W_CDNA4_BLOCKS 1
 
 /* dequant-scale rounding of downcast_to_mxfp (numerics_details/mxfp.py:17-22) */
 #define TAMD_ROUND_UP 0
@@ -266,6 +269,12 @@ typedef struct tamd_matmul_args {
    * y_mx_scale[row, column / 32] (rows placed like the rows of y).  NULL = plain output. */
   uint8_t *y_mx_scale;
   int64_t y_mx_stride_m, y_mx_stride_z;
+  /* encoding of MXFP4 w: TAMD_W_STRIDED (w_stride_* above: K/2 bytes contiguous per column) or TAMD_W_CDNA4_BLOCKS,
+   * this library's own layout (no counterpart in the reference, whose AMD path keeps the strided one;
+   * tensor_details/layout.py CDNA4MXValueLayout): per expert ceil(N/64) strips x ceil(K/128) stages of 4 KB blocks,
+   * K and N padded with zero codes; in a block, column 2c + f of the strip is position 32 f + c (64 bytes), its
+   * 16-byte part p in slot p ^ ((c >> 2) & 3) ^ 2 f.  Only w_stride_e is used (bytes); w 16-byte aligned. */
+  int w_layout;
 } tamd_matmul_args;
 
 int tamd_matmul(const tamd_matmul_args *args, void *stream);

@@ -1,4 +1,6 @@
-"""CPU oracle: the CDNA4 pre-shuffle of MXFP4 weight scales.  Test infrastructure, never shipped.
+"""CPU oracle: the CDNA4 pre-shuffle of MXFP4 weight scales, and the block layout of MXFP4 weight codes that the
+gfx950 kernels read (cdna4_value_*: this build's own wire format, no counterpart in the reference; pinned by its
+definition worked by hand and by the round trip).  Test infrastructure, never shipped.
 
 Restates, with numpy index arithmetic (no reshape / permute chains, so that it shares no code shape with the
 product's torch implementation):
@@ -66,3 +68,49 @@ def cdna4_block_unswizzle_ref(block: np.ndarray, block_n: int, block_k_scale: in
                             out[nb * 32 + n2 * 16 + n16, k8 * 8 + k2 * 4 + k4] = flat[i]
                             i += 1
     return out
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# MXFP4 value layout of the gfx950 kernels: blocks of (64 columns x 128 K) = 4 KB, [strip][K stage][position][slot]
+# ---------------------------------------------------------------------------------------------------------------------
+def cdna4_value_storage_shape(shape):
+    """Logical [..., K, N] (FP4) -> [B, ceil(N/64), ceil(K/128) * 4096] bytes."""
+    *leading, k, n = shape
+    b = int(np.prod(leading)) if leading else 1
+    return [b, -(-n // 64), -(-k // 128) * 4096]
+
+
+def cdna4_value_offset(kb: int, n: int, ks_count: int) -> int:
+    """Byte offset, inside one matrix's storage, of packed byte `kb` (codes 2 kb and 2 kb + 1) of column `n`."""
+    strip, cn = divmod(n, 64)
+    c, f = divmod(cn, 2)            # the column pair (2c, 2c + 1) shares c: positions c and 32 + c
+    ks, within = divmod(kb, 64)     # K stage of 128 codes = 64 bytes
+    part, byte = divmod(within, 16)
+    slot = part ^ ((c >> 2) & 3) ^ (2 * f)
+    return (strip * ks_count + ks) * 4096 + (32 * f + c) * 64 + slot * 16 + byte
+
+
+def cdna4_value_swizzle_ref(x: np.ndarray) -> np.ndarray:
+    """x: uint8 [..., K/2, N] packed codes -> [B, ceil(N/64), ceil(K/128) * 4096]; padding bytes are zero.  Plain
+    loops over every byte (small inputs only)."""
+    *leading, kb_count, n_count = x.shape
+    b, ns, row = cdna4_value_storage_shape([*leading, kb_count * 2, n_count])
+    ks_count = row // 4096
+    out = np.zeros((b, ns * row), dtype=np.uint8)
+    xb = x.reshape(b, kb_count, n_count)
+    for kb in range(kb_count):
+        for n in range(n_count):
+            out[:, cdna4_value_offset(kb, n, ks_count)] = xb[:, kb, n]
+    return out.reshape(b, ns, row)
+
+
+def cdna4_value_unswizzle_ref(stored: np.ndarray, shape) -> np.ndarray:
+    *leading, k, n_count = shape
+    b = stored.shape[0]
+    ks_count = stored.shape[-1] // 4096
+    flat = stored.reshape(b, -1)
+    out = np.zeros((b, k // 2, n_count), dtype=np.uint8)
+    for kb in range(k // 2):
+        for n in range(n_count):
+            out[:, kb, n] = flat[:, cdna4_value_offset(kb, n, ks_count)]
+    return out.reshape(*leading, k // 2, n_count)

@@ -80,12 +80,25 @@ def test_config2_routing(device):
         torch.testing.assert_close(r.vals.cpu(), ref["vals"], rtol=1e-5, atol=1e-6)
 
 
-@pytest.mark.parametrize("scale_layout", ["strided", "cdna4"])
+LAYOUTS = [("strided", "strided"), ("cdna4", "strided"), ("cdna4", "blocks")]
+
+
+def weights_for_matmul(vals, value_layout):
+    """MXFP4 codes as downcast_to_mxfp leaves them (K contiguous per column), or in the kernels' block layout."""
+    if value_layout == "strided":
+        return vals
+    from triton_amd.tensor import FP4, convert_layout, wrap_torch_tensor
+    from triton_amd.tensor_details.layout import CDNA4MXValueLayout
+    return convert_layout(wrap_torch_tensor(vals, dtype=FP4), CDNA4MXValueLayout())
+
+
+@pytest.mark.parametrize("scale_layout,value_layout", LAYOUTS)
 @pytest.mark.parametrize("T", [4096, 64])
-def test_config3_and_4_up_projection(T, scale_layout, device):
+def test_config3_and_4_up_projection(T, scale_layout, value_layout, device):
     """T=4096 (prefill, tiled kernel) and T=64 (decode, streaming kernel): hidden 2880, 128 experts, top-4,
     W1 [128, 2880, 5760] MXFP4, bias + SwiGLU; weight scales strided or in the CDNA4 pre-shuffle (the layout the
-    reference picks on this target, tensor_details/layout.py:43-54)."""
+    reference picks on this target, tensor_details/layout.py:43-54), weight codes strided or in the kernels' block
+    layout."""
     E, k, K, N = 128, 4, 2880, 5760
     torch.manual_seed(0)
     logits = torch.randn(T, E)
@@ -93,31 +106,32 @@ def test_config3_and_4_up_projection(T, scale_layout, device):
     bias = (torch.randn(E, N) * 0.01).to(torch.bfloat16)
     vals, scales = bench.make_weights(E, K, N, device)
     mm_scales = bench.scales_for_matmul(scales, scale_layout)
+    mm_vals = weights_for_matmul(vals, value_layout)
     pc = PrecisionConfig(b_mx_scale=mm_scales, b_microblock_size=32)
     r = routing(logits.to(device), k)
     ref = RR.routing_ref(logits, k)
     assert torch.equal(r.gather_indx.cpu(), ref["gather_indx"]) and torch.equal(r.col_sum.cpu(), ref["col_sum"])
     xd, bd = x.to(device), bias.to(device)
-    y = matmul(xd, vals, bd, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=SWIGLU)
+    y = matmul(xd, mm_vals, bd, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=SWIGLU)
     assert tuple(y.shape) == (T * k, N // 2)
     busiest = int(ref["col_sum"].argmax())
     # every expert with the production layout (about ten seconds of oracle time on the host cores), a sample otherwise
-    experts = range(E) if scale_layout == "cdna4" else sorted({0, 1, 63, 127, busiest})
+    experts = range(E) if value_layout == "blocks" else sorted({0, 1, 63, 127, busiest})
     sample_check(y, x, vals, scales, bias, ref, experts, True)
     # rows that gather the same token into the same expert are impossible (top-k picks distinct experts), but the
     # same token under different experts must differ; the same (token, expert) computed twice must agree exactly
-    y2 = matmul(xd, vals, bd, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=SWIGLU)
+    y2 = matmul(xd, mm_vals, bd, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc, fused_activation=SWIGLU)
     assert torch.equal(y, y2)
     # power-of-two scaling of the activations is exact through the linear part (no activation, no bias)
-    lin = matmul(xd, vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc)
-    lin4 = matmul((x * 4).to(device), vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc)
+    lin = matmul(xd, mm_vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc)
+    lin4 = matmul((x * 4).to(device), mm_vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc)
     assert torch.equal(lin4.float(), lin.float() * 4)
     # one-hot activations return dequantised weight rows bit for bit (float32 output)
     eye = torch.zeros(T, K, dtype=torch.bfloat16)
     hot = torch.randint(0, K, (T, ))
     eye[torch.arange(T), hot] = 1.0
     pc32 = PrecisionConfig(b_mx_scale=mm_scales, b_microblock_size=32, out_dtype=torch.float32)
-    rows = matmul(eye.to(device), vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc32).cpu()
+    rows = matmul(eye.to(device), mm_vals, None, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc32).cpu()
     offs = torch.cat([torch.zeros(1, dtype=torch.int64), ref["col_sum"].long().cumsum(0)])
     for e in (0, 77, busiest):
         lo, hi = int(offs[e]), int(offs[e + 1])
@@ -128,10 +142,10 @@ def test_config3_and_4_up_projection(T, scale_layout, device):
         assert torch.equal(rows[lo:hi], deq[hot[tok]])
 
 
-@pytest.mark.parametrize("scale_layout", ["strided", "cdna4"])
-def test_config5_down_projection_and_combine(scale_layout, device):
+@pytest.mark.parametrize("scale_layout,value_layout", LAYOUTS)
+def test_config5_down_projection_and_combine(scale_layout, value_layout, device):
     """T=16384, 32 experts, top-4: fp8 expert-sorted rows x W2 [32, 2880, 2880] MXFP4, gate weights, scatter, then
-    the top-4 combine; weight scales strided or in the CDNA4 pre-shuffle."""
+    the top-4 combine; weight scales strided or in the CDNA4 pre-shuffle, weight codes strided or in blocks."""
     T, E, k, K, N = 16384, 32, 4, 2880, 2880
     rows = T * k
     torch.manual_seed(0)
@@ -152,12 +166,13 @@ def test_config5_down_projection_and_combine(scale_layout, device):
                          out_dtype=torch.bfloat16,
                          flex_ctx=FlexCtx(lhs_data=InFlexData(dtype=torch.float8_e4m3fn, scale=x_scale)))
     bd = bias.to(device)
-    y_sorted = matmul(x8, vals, bd, r.ragged_metadata, precision_config=pc, gammas=gam)
-    y = matmul(x8, vals, bd, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam)
+    mm_vals = weights_for_matmul(vals, value_layout)
+    y_sorted = matmul(x8, mm_vals, bd, r.ragged_metadata, precision_config=pc, gammas=gam)
+    y = matmul(x8, mm_vals, bd, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc, gammas=gam)
     # the scattered result is the expert-sorted one, permuted
     assert torch.equal(y[r.scatter_indx.long()], y_sorted)
     busiest = int(ref["col_sum"].argmax())
-    experts = range(E) if scale_layout == "cdna4" else sorted({0, 31, busiest})
+    experts = range(E) if value_layout == "blocks" else sorted({0, 31, busiest})
     sample_check(y_sorted, x8.cpu(), vals, scales, bias, ref, experts, False, sorted_x=True,
                  x_scale=x_scale.cpu(), gammas=gam.cpu())
     z, _ = reduce(y.view(T, k, N), dim=1)

@@ -15,8 +15,8 @@ from triton_amd.matmul import FlexCtx, FnSpecs, FusedActivation, InFlexData, Pre
 from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
 from triton_amd.numerics_details.mxfp import downcast_to_mxfp
 from triton_amd.swiglu import swiglu_fn
-from triton_amd.tensor import convert_layout, make_ragged_tensor_metadata, wrap_torch_tensor
-from triton_amd.tensor_details.layout import CDNA4MXScaleLayout
+from triton_amd.tensor import FP4, convert_layout, make_ragged_tensor_metadata, wrap_torch_tensor
+from triton_amd.tensor_details.layout import CDNA4MXScaleLayout, CDNA4MXValueLayout
 from triton_amd.testing import assert_close
 
 pytestmark = pytest.mark.gpu
@@ -41,7 +41,14 @@ def make_case(seed):
     c["bias"] = rng.choice([None, torch.float32, torch.bfloat16, torch.float16])
     c["act"] = rng.random() < 0.5
     c["out"] = rng.choice([None, torch.float32]) if c["kind"] in ("bf16", "f16") else rng.choice([torch.bfloat16, torch.float32])
+    # weight codes in the kernels' block layout (a generator of its own: the other choices keep their sequence)
+    c["blocks"] = random.Random(7777 + seed).random() < 0.5
     return c
+
+
+def in_blocks(v):
+    """MXFP4 codes as downcast_to_mxfp returns them -> the kernels' block layout."""
+    return convert_layout(wrap_torch_tensor(v, dtype=FP4), CDNA4MXValueLayout())
 
 
 # TAMD_SWEEP_CASES widens the sweep for exploration; the default keeps the suite short
@@ -105,7 +112,7 @@ def test_sweep(seed, device):
     fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if c["act"] else None
     out_init = torch.zeros((M, N // 2 if c["act"] else N), dtype=out_dtype, device=device)
     with scoped_opt_flags_constraints({} if c["block_m"] is None else {"block_m": c["block_m"]}):
-        out = matmul(xdev, v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter), precision_config=pc,
+        out = matmul(xdev, in_blocks(v) if c["blocks"] else v, dev(bias), md, gather_indx=dev(gather), scatter_indx=dev(scatter), precision_config=pc,
                      betas=dev(betas), gammas=dev(gammas), fused_activation=fa, c=out_init)
     ref = ref.to(out_dtype)
     torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
@@ -152,6 +159,8 @@ def test_sweep_dense_and_batched(seed, device):
         rv, rs = downcast_to_mxfp_ref(w, torch.uint8, axis=-2)
         assert torch.equal(v.cpu(), rv) and torch.equal(s.cpu(), rs)
         wdev, kw["b_mx_scale"] = v, rs
+        if c["split_k"] == 1 and random.Random(8888 + seed).random() < 0.5:
+            wdev = in_blocks(v)  # the kernels' block layout (split_k needs the strided one)
         sc = convert_layout(wrap_torch_tensor(s), CDNA4MXScaleLayout()) if c["cdna4"] else s
         wref = rv
     else:
@@ -237,10 +246,12 @@ def test_sweep_quantised_outputs(seed, device):
     fa = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.702, 7.0)) if act else None
     n_out = N // 2 if act else N
 
+    wq = in_blocks(v) if seed % 2 else v
+
     def run(pc, **kw):
         out_init = torch.zeros((M, n_out), dtype=pc.out_dtype, device=device)
         with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
-            return matmul(xdev, v, bias, md, scatter_indx=scatter, precision_config=pc, gammas=gammas, fused_activation=fa,
+            return matmul(xdev, wq, bias, md, scatter_indx=scatter, precision_config=pc, gammas=gammas, fused_activation=fa,
                           c=out_init, **kw)
 
     y32 = run(PrecisionConfig(b_mx_scale=sc, b_microblock_size=32, out_dtype=torch.float32, flex_ctx=FlexCtx(lhs_data=lhs))).cpu()

@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("TAMD_LIB") or os.path.join(_HERE, "libtriton_amd.so")
 F32, F16, BF16, FP8_E4M3, FP8_E5M2, MXFP4 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_SWIGLU = 0, 1
 SCALE_STRIDED, SCALE_CDNA4 = 0, 1
+W_STRIDED, W_CDNA4_BLOCKS = 0, 1
 E_INVALID, E_UNSUPPORTED, E_ALIGNMENT, E_TOO_LARGE = -1, -2, -3, -4
 
 _TORCH_CODE = {
@@ -54,6 +55,7 @@ class MatmulArgs(C.Structure):
         ("w_mx_layout", C.c_int),
         ("x_mx_scale", C.c_void_p), ("x_mx_stride_m", C.c_int64), ("x_mx_stride_z", C.c_int64),
         ("y_mx_scale", C.c_void_p), ("y_mx_stride_m", C.c_int64), ("y_mx_stride_z", C.c_int64),
+        ("w_layout", C.c_int),
     ]
 
 

@@ -41,6 +41,28 @@ def _scratch_users(remarks):
     return out
 
 
+def _scratch_instructions(src, names):
+    """Number of scratch loads / stores in the generated code of the kernels `names` of one source (the device
+    assembly is produced for this check only)."""
+    asm = os.path.join(HERE, "build", os.path.splitext(src)[0] + ".check.s")
+    cmd = [HIPCC, *FLAGS, *EXTRA, "-x", "hip", "--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", asm]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        return {}
+    counts, cur = {}, None
+    with open(asm) as f:
+        for line in f:
+            if line and not line[0].isspace() and line.rstrip().split(":")[0] in names and ":" in line:
+                cur = line.split(":")[0]
+                counts.setdefault(cur, 0)
+            elif ".end_amdhsa_kernel" in line:
+                cur = None
+            elif cur is not None and re.search(r"\bscratch_(load|store)", line):
+                counts[cur] += 1
+    os.remove(asm)
+    return counts
+
+
 def _compile(src, obj):
     cmd = [HIPCC, *FLAGS, *EXTRA, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
     if src.endswith(".hip"):
@@ -51,6 +73,11 @@ def _compile(src, obj):
     # every kernel here is written to live in registers; one that falls into scratch memory still computes
     # the right values, several times slower, so the build is where it has to be caught
     spilled = _scratch_users(res.stderr)
+    if spilled and not os.environ.get("TAMD_ALLOW_SCRATCH"):
+        # a kernel may be given a small private segment without a single access to it (stack slots the register
+        # allocator reserved and then did not need): what counts is whether its code touches scratch memory
+        touching = _scratch_instructions(src, [n for n, _ in spilled])
+        spilled = [(n, b) for n, b in spilled if touching.get(n, 1) > 0]
     if spilled and not os.environ.get("TAMD_ALLOW_SCRATCH"):
         os.remove(obj)
         raise RuntimeError(f"{src}: kernels using scratch memory: " + ", ".join(f"{n} ({b} B/lane)" for n, b in spilled))

@@ -43,6 +43,13 @@ extern "C" int tamd_matmul(const tamd_matmul_args *args, void *stream) {
     // weights / scales must be contiguous along K ("column-major" mxfp weights)
     const bool cdna4_sc = a.w_mx_layout == TAMD_SCALE_CDNA4;
     if (a.w_mx_layout != TAMD_SCALE_STRIDED && !cdna4_sc) return TAMD_E_INVALID;
+    const bool w_blocks = a.w_layout == TAMD_W_CDNA4_BLOCKS;
+    if (a.w_layout != TAMD_W_STRIDED && !w_blocks) return TAMD_E_INVALID;
+    if (w_blocks) {
+      // only the expert pitch is used; a matrix is ceil(N/64) x ceil(K/128) blocks of 4 KB
+      a.w_stride_k = 1, a.w_stride_n = 0;
+      if ((int64_t)((a.N + 63) / 64) * ((a.K + 127) / 128) * 4096 >= (int64_t)0x7FFFFF00) return TAMD_E_UNSUPPORTED;
+    }
     if (a.w_stride_k != 1 || (!cdna4_sc && a.w_mx_stride_k != 1)) return TAMD_E_UNSUPPORTED;
     if (cdna4_sc && (!aligned(a.w_mx_scale, 16) || a.w_mx_stride_e % 16 != 0)) return TAMD_E_ALIGNMENT;
     if (!aligned(a.w, 16) || a.w_stride_n % 16 != 0 || a.w_stride_e % 16 != 0) return TAMD_E_ALIGNMENT;

@@ -257,8 +257,9 @@ constexpr PipeShape pipe_shape(bool fp8, bool ring, int lds_rows) {
 // 160 x 256 of them.  The element loops must unroll completely (the accumulators are indexed by them and
 // would otherwise live in scratch memory), and the compiler gives up on that above a body size that one
 // variant holding every feature exceeds: hence MXO and FLEX exclude each other.
-template <int NFR, int ACT, int YDT, bool ROWSC, bool FLEX, bool MXO = false>
-TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
+// Args: tamd_matmul_args, or the same structure read in place from the kernel-argument segment (see kernel_args_late).
+template <int NFR, int ACT, int YDT, bool ROWSC, bool FLEX, bool MXO = false, typename Args = tamd_matmul_args>
+TAMD_DEVICE void tile_epilogue_t(const Args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
   const int c32 = lane % 32, h = lane / 32;
@@ -533,19 +534,31 @@ TAMD_DEVICE void tile_epilogue_t(const tamd_matmul_args &a, const Tile &t, f32x1
 // activations); any other combination takes the general one.
 // FP8_ROWS: the kernel's activations are fp8; then a plain float8_e4m3fn output (the rows the next matmul of an
 // MoE layer consumes) is specialised as well.
-template <int NFR, int ACT, int FAST_YDT, bool FP8_ROWS>
-TAMD_DEVICE void tile_epilogue(const tamd_matmul_args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
+template <int NFR, int ACT, int FAST_YDT, bool FP8_ROWS, typename Args>
+TAMD_DEVICE void tile_epilogue(const Args &a, const Tile &t, f32x16_t (&acc)[NFR][NF], uint8_t *lds) {
   const bool flexo = a.y_expected_scale != nullptr || a.y_actual_scale != nullptr;
   if (a.y_mx_scale) {  // always e4m3 values and no flexpoint output (checked by the entry point)
-    tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false, true>(a, t, acc, lds);
+    tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false, true, Args>(a, t, acc, lds);
   } else if (FP8_ROWS && a.y_dtype == TAMD_FP8_E4M3 && !flexo) {
-    if constexpr (FP8_ROWS) tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false>(a, t, acc, lds);
+    if constexpr (FP8_ROWS) tile_epilogue_t<NFR, ACT, TAMD_FP8_E4M3, true, false, false, Args>(a, t, acc, lds);
   } else if (a.y_dtype == FAST_YDT && !flexo) {
-    if (a.betas || a.gammas) tile_epilogue_t<NFR, ACT, FAST_YDT, true, false>(a, t, acc, lds);
-    else tile_epilogue_t<NFR, ACT, FAST_YDT, false, false>(a, t, acc, lds);
+    if (a.betas || a.gammas) tile_epilogue_t<NFR, ACT, FAST_YDT, true, false, false, Args>(a, t, acc, lds);
+    else tile_epilogue_t<NFR, ACT, FAST_YDT, false, false, false, Args>(a, t, acc, lds);
   } else {
-    tile_epilogue_t<NFR, ACT, -1, true, true>(a, t, acc, lds);
+    tile_epilogue_t<NFR, ACT, -1, true, true, false, Args>(a, t, acc, lds);
   }
+}
+
+// The kernel's tamd_matmul_args (its first parameter) read in place from the kernel-argument segment, through a
+// pointer the compiler cannot see through.  The compiler loads every field of a by-value kernel argument that is
+// used anywhere into scalar registers at the top of the kernel; the few dozen that only the epilogue needs then
+// stay live through the K loop, the scalar registers overflow into vector registers, and a kernel that sits at 256
+// of those starts spilling accumulators.  Read this way, the epilogue's fields are fetched when it begins.
+typedef const __attribute__((address_space(4))) tamd_matmul_args late_args_t;
+TAMD_DEVICE late_args_t &kernel_args_late() {
+  late_args_t *p = (late_args_t *)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(p));
+  return *p;
 }
 
 // One output tile with NFR (compile time) active 32-row fragments.
@@ -686,14 +699,24 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     a_off[i] = r < t.rows ? src * (uint32_t)(a.x_stride_m * ESZ) + a_chunk * 16 : kOob;
   }
   // ---- weight DMA: instruction j copies LDS positions j*16 + lane/4, part slot lane%4
+  // Codes in the block layout (TAMD_W_CDNA4_BLOCKS): a stage of this wave's strip is one 4 KB block that already has
+  // the LDS image's order, so the four copies are linear (whole, aligned lines) and the K stage enters through the
+  // scalar offset; K and N are padded with zero codes, nothing is masked.
+  const bool wnat = a.w_layout == TAMD_W_CDNA4_BLOCKS;
+  const int w_stage_shift = wnat ? 12 : 6;   // bytes from one K stage to the next: a 4 KB block, or 64 bytes of a column
+  // (the lane's 16-byte part of a column is the same for copies 0, 1 and, two further on, for copies 2, 3:
+  // (pos >> 2) & 3 = (lane / 16) & 3 for every j, (pos >> 5) << 1 = 2 (j / 2))
   uint32_t w_off[4];
-  int w_part[4];
+  const int w_part0 = (lane % 4) ^ ((lane / 16) & 3);
+  const int w_kpart0 = wnat ? 0 : w_part0 * 32;   // K offset (codes) of the lane's bytes inside a stage; block layout: padded, 0
+  auto w_kpart = [&](int j) { return wnat ? 0 : (w_kpart0 ^ ((j >> 1) << 6)); };
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int pos = j * 16 + lane / 4;  // f*32 + c
     const int col = t.n0 + wave * 64 + 2 * (pos % 32) + pos / 32;
-    w_part[j] = (lane % 4) ^ ((pos >> 2) & 3);
-    w_off[j] = (uint32_t)(col < N ? col : N - 1) * (uint32_t)a.w_stride_n + w_part[j] * 16;
+    const int part = w_part0 ^ ((j >> 1) << 1);
+    w_off[j] = wnat ? (uint32_t)(((t.n0 >> 6) + wave) * ((K + KB - 1) / KB)) * 4096u + (uint32_t)(j * 1024 + lane * 16)
+                    : (uint32_t)(col < N ? col : N - 1) * (uint32_t)a.w_stride_n + part * 16;
   }
   // ---- this lane's MFMA columns
   const int col0 = t.n0 + wave * 64 + c32 * NF;
@@ -722,8 +745,8 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     const int kb = sup * KB;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t bkill = (wave_live && kb + w_part[j] * 32 < K) ? 0u : kOob;
-      dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, kb >> 1);
+      const uint32_t bkill = (wave_live && kb + w_kpart(j) < K) ? 0u : kOob;
+      dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, (uint32_t)sup << w_stage_shift);
     }
   };
   // Paired form (ring mode, row blocks of up to 64 rows): the weights of stages 2p and 2p + 1 are 128 contiguous bytes
@@ -749,6 +772,15 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   auto issue_b_pair = [&](int pair) {
     if constexpr (PAIRED) {
       const int kb = pair * 256;
+      if (wnat) {
+        // block layout: the pair's two stages are two 4 KB blocks, copied as they lie (first stage, then second)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t bkill = (wave_live && kb + (j >> 2) * KB < K) ? 0u : kOob;
+          dma16(rw, lds_b2 + j * 1024, w_off[j & 3] | bkill, (uint32_t)(2 * pair + (j >> 2)) * 4096u);
+        }
+        return;
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const uint32_t bkill = (wave_live && kb + w2_part[j] * 32 < K) ? 0u : kOob;
@@ -802,11 +834,13 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int pos = f * 32 + c32;
+        const int rot = ((pos >> 2) & 3) ^ (f << 1);   // slot of part p of position pos: p ^ rot
         if constexpr (PAIRED)
-          raw[set][f][q] = *(const uint4 *)(bbuf2 + pos * 128 + (((4 * (sup & 1) + 2 * q + h) ^ ((pos >> 1) & 7)) * 16));
+          raw[set][f][q] = wnat ? *(const uint4 *)(bbuf2 + (sup & 1) * 4096 + pos * 64 + (((2 * q + h) ^ rot) * 16))
+                                : *(const uint4 *)(bbuf2 + pos * 128 + (((4 * (sup & 1) + 2 * q + h) ^ ((pos >> 1) & 7)) * 16));
         else
           raw[set][f][q] = *(const uint4 *)(bbuf + (DB == 2 ? (sup & 1) * B_BYTES : 0) + pos * 64 +
-                                            (((2 * q + h) ^ ((pos >> 2) & 3)) * 16));
+                                            (((2 * q + h) ^ rot) * 16));
         // group kg = 4*sup + 2q + h of this lane's column.  Strided: byte kg, kept inside the column's G bytes
         // (groups past the end of K meet zero codes and zero activations; their scale only has to be some finite
         // value of this column).  Pre-shuffled: byte 256*(kg/8) + 64*(kg%4) + 2*((kg%8)/4); the padding up to a
@@ -866,21 +900,30 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       // one stage = 128 K = two scaled MFMAs per (row fragment, column fragment); the fragments of the first half
       // and the activations' scale operands are already in registers (fp8_read0)
       constexpr int CBSZ = XDT == TAMD_FP8_E5M2 ? 1 : 0;
+      // (the fragments of the second half are requested one by one behind the last MFMAs that use those of the first:
+      // both halves of all fragments at once are 64 registers, which this kernel does not have)
+      const int swz = (c32 >> 1) & 7;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        if (s == 0) fp8_read_frags(buf, 1, af8[1]);
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           const uint4 r = raw[set][f][s];
           const i32x8_t bf = i32x8_t{(int)r.x, (int)r.y, (int)r.z, (int)r.w, 0, 0, 0, 0};
 #pragma unroll
           for (int i = 0; i < NFR; ++i) {
-            if (s == 0)
+            if (s == 0) {
               acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[0][i], bf, acc[i][f], CBSZ, 4, 0, sa8[i], 0,
                                                                         (int)scw[set][f]);
-            else
+              if (f == NF - 1) {
+                const uint8_t *row = buf + (i * 32 + c32) * A_ROW_BYTES;
+                const uint4 lo = *(const uint4 *)(row + (((4 + h) ^ swz) * 16));
+                const uint4 hi = *(const uint4 *)(row + (((6 + h) ^ swz) * 16));
+                af8[1][i] = i32x8_t{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+              }
+            } else {
               acc[i][f] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af8[1][i], bf, acc[i][f], CBSZ, 4, 2, sa8[i], 1,
                                                                         (int)scw[set][f]);
+            }
           }
         }
       }
@@ -1001,7 +1044,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   wait_dma();
 
-  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT, FP8>(a, t, acc, lds);
+  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT, FP8>(kernel_args_late(), t, acc, lds);
 }
 
 // Row fragments a workgroup can hold: a 128-row block of 16-bit activations also takes a remainder of

@@ -288,8 +288,14 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
 #pragma unroll
       for (int q = 1; q < S::NSC; ++q) x_voff[q] = kOob;
     }
+    // codes in the block layout (TAMD_W_CDNA4_BLOCKS): the unit's 16 columns are, in every K stage's 4 KB block of
+    // their strip, two runs of 512 bytes (positions 8u.. and 32 + 8u.., u = unit inside the strip): piece i of the
+    // image is K stage i, lanes 0-31 copy the first run and lanes 32-63 the second
+    const bool wnat = a.w_layout == TAMD_W_CDNA4_BLOCKS;
+    const int n_kstage = (K + 127) / 128;
+    const uint32_t nat_voff = (uint32_t)((lane / 32) * 2048 + (lane % 32) * 16);
     int i_blk = blk0 - 1, i_cg = cg0, i_left = total_stages;
-    uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0;
+    uint32_t i_wbase = 0, i_sbase = 0, i_bbase = 0, i_ebase = 0;
     auto issue = [&](int slot) {
       const bool live = i_left > 0;
       if (live && (i_blk < blk0 || i_cg == n_cg)) {
@@ -298,12 +304,21 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         Block b;
         get_block(i_blk, b);
         const int e = __builtin_amdgcn_readfirstlane(b.expert);  // keeps the running offsets in scalar registers
-        i_wbase = (uint32_t)((int64_t)e * a.w_stride_e) + (uint32_t)i_cg * 16u * col_bytes;
+        i_ebase = (uint32_t)((int64_t)e * a.w_stride_e);
+        i_wbase = i_ebase + (uint32_t)i_cg * 16u * col_bytes;
         i_sbase = (uint32_t)((int64_t)e * a.w_mx_stride_e);
         i_bbase = (uint32_t)(((int64_t)e * a.bias_stride_e + i_cg * 16) * bias_esz);
       }
       const uint32_t sb = lds_base + slot * S::STAGE;
       const v4i_t dw = live ? rw : rw0;
+      if (wnat) {
+        const uint32_t ub = i_ebase + (uint32_t)((i_cg >> 2) * n_kstage) * 4096u + (uint32_t)(i_cg & 3) * 512u;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+          const int ks = half * NP + i;
+          dma16_at<0, true>(ks < n_kstage ? dw : rw0, sb + ks * 1024, nat_voff, ub + (uint32_t)ks * 4096u);
+        }
+      } else
 #pragma unroll
       for (int i = 0; i < NP; ++i) {
         const uint32_t m0v = sb + (half * NP + i / 4 * 4) * 1024;
@@ -404,13 +419,18 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
     };
     // per-lane LDS offsets of this wave's K slice inside a stage (beyond K: group 0 with scale 1.0 --
     // the activations there are zero, the weight operand only has to stay finite)
+    const bool wnat = a.w_layout == TAMD_W_CDNA4_BLOCKS;
     uint32_t b_loff[SS], s_loff[SS];
     bool kvalid[SS];
 #pragma unroll
     for (int j = 0; j < SS; ++j) {
       const int kg = kb + 4 * j + g;
       kvalid[j] = kg < G;
-      b_loff[j] = (uint32_t)c16 * col_bytes + (kvalid[j] ? kg : 0) * 16;
+      // block layout: stage kg / 4 of the image, run f = column parity, position c' = column / 2, the group's part
+      // in slot part ^ (c' >> 2) ^ 2 f (^ 2 for the odd units of a strip, applied per unit below)
+      const int kgv0 = kvalid[j] ? kg : 0, cf = c16 & 1, cp = c16 >> 1;
+      b_loff[j] = wnat ? (uint32_t)((kgv0 >> 2) * 1024 + cf * 512 + cp * 64 + (((kgv0 & 3) ^ (cp >> 2) ^ (cf << 1)) * 16))
+                       : (uint32_t)c16 * col_bytes + kgv0 * 16;
       const int kgv = kvalid[j] ? kg : 0;
       s_loff[j] = (uint32_t)(S::CODE_BYTES +
                              (cdna4 ? (kgv / 8) * 256 + (kgv % 4) * 64 + c16 * 4 + ((kgv % 8) / 4) * 2 : c16 * G + kgv));
@@ -424,13 +444,14 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         load_block(++c_blk);
       }
       const uint32_t sc_par = cdna4 ? (uint32_t)(c_cg & 1) : 0u;  // which 16 of the block's 32 columns
+      const uint32_t b_flip = wnat ? (uint32_t)(c_cg & 1) << 5 : 0u;  // odd unit of a strip: slots rotated by 2
       ++c_cg;
       const uint8_t *img = lds + slot * S::STAGE;
       uint4 raw[SS];
       uint32_t sby[SS];
 #pragma unroll
       for (int j = 0; j < SS; ++j) {
-        raw[j] = *(const uint4 *)(img + b_loff[j]);
+        raw[j] = *(const uint4 *)(img + (b_loff[j] ^ b_flip));
         sby[j] = img[s_loff[j] + sc_par];
       }
       // four independent accumulation chains keep dependent MFMAs apart
@@ -458,10 +479,11 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   const int64_t G = a.K / 32;
   if (a.K > 4096 || a.K % 32 != 0) return false;
   const bool cdna4 = a.w_mx_layout == TAMD_SCALE_CDNA4;
-  if (a.w_stride_k != 1 || a.w_stride_n != a.K / 2) return false;
+  const bool wnat = a.w_layout == TAMD_W_CDNA4_BLOCKS;
+  if (!wnat && (a.w_stride_k != 1 || a.w_stride_n != a.K / 2)) return false;
   if (!cdna4 && (a.w_mx_stride_k != 1 || a.w_mx_stride_n != G)) return false;
   if (!aligned(a.w, 16) || a.w_stride_e % 16 != 0 || !aligned(a.w_mx_scale, 16) || a.w_mx_stride_e % 16 != 0) return false;
-  if ((int64_t)a.n_experts * a.w_stride_e + (int64_t)a.N * a.w_stride_n >= lim) return false;
+  if ((int64_t)a.n_experts * a.w_stride_e + (wnat ? (int64_t)0 : (int64_t)a.N * a.w_stride_n) >= lim) return false;
   if ((int64_t)a.n_experts * a.w_mx_stride_e + (int64_t)(a.N + 32) * (G + 8) >= lim) return false;
   if (a.bias && ((int64_t)a.n_experts * a.bias_stride_e + a.N) * 4 >= lim) return false;
   if (a.bias && !aligned(a.bias, a.bias_dtype == TAMD_F32 ? 4 : 2)) return false;

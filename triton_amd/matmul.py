@@ -17,7 +17,7 @@ from .matmul_details.opt_flags import (InapplicableConstraint, OptFlags, make_op
 from .numerics import InFlexData, OutFlexData
 from .specialize import FnSpecs
 from .tensor import FP4, RaggedTensorMetadata, Tensor, wrap_torch_tensor
-from .tensor_details.layout import CDNA4MXScaleLayout
+from .tensor_details.layout import CDNA4MXScaleLayout, CDNA4MXValueLayout
 
 __all__ = ["matmul", "matmul_ogs", "PrecisionConfig", "FlexCtx", "FusedActivation", "Epilogue", "FnSpecs",
            "InFlexData", "OutFlexData", "InapplicableConstraint", "OptFlags", "scoped_opt_flags",
@@ -170,6 +170,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     # ---- weights
     b_scale = precision_config.b_mx_scale
     # weights: storage tensor, whether they are packed e2m1 codes, logical shape (a packed axis counts twice)
+    b_blocks = isinstance(b, Tensor) and isinstance(b.storage.layout, CDNA4MXValueLayout)  # the kernels' own value layout
     if isinstance(b, Tensor):
         b_data, b_fp4, b_shape = b.storage.data, b.dtype == FP4, list(b.shape)
     else:
@@ -291,7 +292,16 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         args.x_mx_scale = a_mx_scale.data_ptr()
         args.x_mx_stride_m = a_mx_scale.stride(-2)
         args.x_mx_stride_z = a_mx_scale.stride(0) if a_mx_scale.ndim == 3 else 0
-    wd = w if w.ndim == 3 else w[None]
+    if b_blocks:
+        # storage [B, ceil(N/64), ceil(K/128) * 4096]: strips of 4 KB blocks, one matrix after the other
+        assert b_fp4 and w.ndim == 3 and w.is_contiguous(), "block-layout weights are packed e2m1 codes"
+        want_b = math.prod(b_shape[:-2])
+        assert list(w.shape) == CDNA4MXValueLayout().storage_shape([want_b, K_W, N]), \
+            f"storage {tuple(w.shape)} does not match the block layout of weights {b_shape}"
+        args.w_layout = _lib.W_CDNA4_BLOCKS
+        wd = w
+    else:
+        wd = w if w.ndim == 3 else w[None]
     args.w = wd.data_ptr()
     if b_fp4:
         assert b_scale is not None, "MXFP4 weights need precision_config.b_mx_scale"
@@ -314,7 +324,10 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
             args.w_mx_stride_e, args.w_mx_stride_k, args.w_mx_stride_n = sd.stride()
     else:
         args.w_dtype = _lib.dtype_code(w.dtype)
-    args.w_stride_e, args.w_stride_k, args.w_stride_n = wd.stride()
+    if b_blocks:
+        args.w_stride_e, args.w_stride_k, args.w_stride_n = wd.stride(0), 1, 0
+    else:
+        args.w_stride_e, args.w_stride_k, args.w_stride_n = wd.stride()
     args.w_scale = None if flex.rhs_data.scale is None else flex.rhs_data.scale.data_ptr()
     if bias is not None:
         bb = bias if bias.ndim == 2 else bias[None]
@@ -369,7 +382,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if (split_k == 1 and _opt_flags._constraints().get("split_k") is None and _opt_flags._opt_flags.get() is None
             and not ragged and batch == 1 and M <= 256 and K >= 8192 and scatter_indx is None and not mx_out
             and not args.y_expected_scale and not args.y_actual_scale and out.dtype.itemsize > 1
-            and args.w_mx_layout != _lib.SCALE_CDNA4):
+            and args.w_mx_layout != _lib.SCALE_CDNA4 and not b_blocks):
         # few rows and a long K: a tile's K loop is bound by the latency of its stages and there are too few
         # tiles to hide it, so the ranges of a split run side by side (16 x 16384 x 512: 144 us -> 50 us)
         split_k = next((s for s in (8, 4, 2) if K % (s * 128) == 0 and K // s >= 1024), 1)
@@ -395,8 +408,8 @@ def _matmul_split_k(args, split_k, a, wd, w_is_fp4, out, fused_activation, bias,
     from .reduce import reduce
     if args.scatter_indx or args.y_mx_scale:
         raise InapplicableConstraint("split_k cannot be combined with a scatter or a microscaled output")
-    if args.w_mx_layout == _lib.SCALE_CDNA4:
-        raise InapplicableConstraint("split_k needs weight scales in the strided layout")
+    if args.w_mx_layout == _lib.SCALE_CDNA4 or args.w_layout == _lib.W_CDNA4_BLOCKS:
+        raise InapplicableConstraint("split_k needs weights and weight scales in the strided layouts")
     K, N = args.K, args.N
     if not w_is_fp4 and K % 64 != 0:
         # the kernel for 16-bit weights bounds its K tail by the end of the expert's weights, which a range

@@ -10,7 +10,7 @@ from .tensor_details import bitmatrix as _bitmatrix
 from .tensor_details import ragged_tensor as _ragged
 from .tensor_details.dtype import (BF16, BIT, FP4, FP8_E4M3FN, FP8_E4M3FNUZ, FP8_E5M2, FP16, FP32, FP64, INT16,
                                    INT32, INT64, UINT8, DataType, FloatType, IntegerType)
-from .tensor_details.layout import CDNA4MXScaleLayout, Layout, StridedLayout
+from .tensor_details.layout import CDNA4MXScaleLayout, CDNA4MXValueLayout, Layout, StridedLayout
 from .tensor_details.ragged_tensor import RaggedTensorMetadata
 from .tensor_details.bitmatrix import BitmatrixMetadata
 
@@ -144,6 +144,17 @@ def convert_layout(tensor: Tensor, layout: Layout) -> Tensor:
     """Re-encodes `tensor` in `layout`: another contiguous (packed) axis, or the CDNA4 scale pre-shuffle and back
     (reference tensor.py:235-252).  Returns `tensor` itself when its storage already has that encoding."""
     src = tensor.storage.layout
+    if isinstance(src, CDNA4MXValueLayout) or isinstance(layout, CDNA4MXValueLayout):
+        if src == layout:
+            return tensor
+        assert tensor.dtype == FP4, "the CDNA4 value layout holds packed e2m1 codes"
+        if isinstance(src, CDNA4MXValueLayout):
+            data = src.make_transformation(tensor.shape).unswizzle_data(tensor.storage.data)   # unit stride along K
+            strided = Tensor(Storage(data, StridedLayout(-2)), dtype=FP4, shape=list(tensor.shape))
+            return convert_layout(strided, layout)
+        k_major = convert_layout(tensor, StridedLayout(-2))   # packed along K, whatever the source packs along
+        data = layout.make_transformation(tensor.shape).swizzle_data(k_major.storage.data)
+        return Tensor(Storage(data, layout), dtype=FP4, shape=list(tensor.shape))
     if isinstance(src, CDNA4MXScaleLayout) or isinstance(layout, CDNA4MXScaleLayout):
         if src == layout:
             return tensor
