@@ -53,6 +53,8 @@ WORKLOADS = {
     # weights): gate matmul -> top-k + softmax -> metadata -> FC1 + SwiGLU (gathered rows) -> FC2 (rows scattered back
     # to token order) -> sum over the k slots
     "mlp": dict(bpe=64, dim1=5760, dim2=5760, E=128, k=4, mlp=True),
+    # every point of that sweep (bench_mlp.py:256: 1, 2, 4, ... 64 rows per expert), weights made once
+    "mlp_sweep": dict(bpe=[1, 2, 4, 8, 16, 32, 64], dim1=5760, dim2=5760, E=128, k=4, mlp=True),
     # not a path workload: a plain elementwise copy of known size, the yardstick the HBM counters
     # (FETCH_SIZE / WRITE_SIZE) and the achievable copy bandwidth are calibrated with
     "hbm_copy": dict(bytes=1 << 30),
@@ -600,7 +602,9 @@ def run_fc1(args, cfg, name):
 def run_mlp(args, cfg, name):
     """bench/bench_mlp.py:60-96 of the reference with one rank: every stage is timed with HIP events, and checked
     against the oracle given the GPU's own output of the stage before (logits -> routing, bit-exact; FC1 and FC2 on a
-    sample of experts, within the fp8 output step; the combine, bit-exact)."""
+    sample of experts, within the fp8 output step; the combine, bit-exact).  `cfg["bpe"]` may be one number of rows
+    per expert or the list of the reference's sweep (bench_mlp.py:256: 1 ... 64); the weights are made once, the
+    line describes the last (largest) point and carries every point under "sweep"."""
     from oracle import matmul_ref as MR
     from oracle import routing_ref as RR
     from triton_amd.matmul import FnSpecs, FusedActivation, PrecisionConfig, matmul
@@ -609,7 +613,7 @@ def run_mlp(args, cfg, name):
     from triton_amd.swiglu import swiglu_fn
     from triton_amd.numerics_details.mxfp import downcast_to_mxfp
     E, k, d1, d2 = cfg["E"], cfg["k"], cfg["dim1"], cfg["dim2"]
-    T = cfg["bpe"] * E // k
+    bpes = [args.bpe] if args.bpe else (cfg["bpe"] if isinstance(cfg["bpe"], (list, tuple)) else [cfg["bpe"]])
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev)
     g.manual_seed(0)
@@ -630,99 +634,129 @@ def run_mlp(args, cfg, name):
         return vals, scales
     w1, s1 = quantise(d1, d2)
     w2, s2 = quantise(d2 // 2, d1)
-    x8 = rnd(T, d1).to(torch.float8_e4m3fn)
-    x16 = x8.to(torch.bfloat16)
     w1q, w2q = weights_for_matmul(w1, args.value_layout), weights_for_matmul(w2, args.value_layout)
     pc1 = PrecisionConfig(b_mx_scale=scales_for_matmul(s1, args.scale_layout), b_microblock_size=32)
     pc2 = PrecisionConfig(b_mx_scale=scales_for_matmul(s2, args.scale_layout), b_microblock_size=32)
     act1 = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.0, 1.0))
     names = ("gate_matmul", "routing", "fc1_swiglu", "fc2_scatter", "combine")
 
-    def step(ev=None):
-        mark = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
-        mark(0)
-        logits = matmul(x16, wg, bg)
-        mark(1)
-        r = routing(logits, k)
-        mark(2)
-        y1 = matmul(x8, w1q, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
-        mark(3)
-        y2 = matmul(y1, w2q, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
-        mark(4)
-        z, _ = reduce(y2.view(T, k, d1), dim=1)
-        mark(5)
-        return logits, r, y1, y2, z
+    def point(bpe):
+        T = bpe * E // k
+        x8 = rnd(T, d1).to(torch.float8_e4m3fn)
+        x16 = x8.to(torch.bfloat16)
 
-    spin_up(step)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        logits, r, y1, y2, z = step(events[i])
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    stage_ms = {n: median([e[i].elapsed_time(e[i + 1]) for e in events]) for i, n in enumerate(names)}
-    rows = T * k
-    flops = {"gate_matmul": 2.0 * T * d1 * E, "fc1_swiglu": 2.0 * rows * d1 * d2, "fc2_scatter": 2.0 * rows * (d2 // 2) * d1}
-    n_active = int((r.col_sum > 0).sum())
-    w_bytes = lambda K, N: n_active * (K // 2 * N + K // 32 * N + N * 4)
-    bytes_ = {"gate_matmul": T * d1 * 2 + d1 * E * 2 + T * E * 2, "fc1_swiglu": rows * d1 + w_bytes(d1, d2) + rows * d2 // 2,
-              "fc2_scatter": rows * d2 // 2 + w_bytes(d2 // 2, d1) + rows * d1, "combine": rows * d1 + T * d1}
-    stages = {}
-    for n in names:
-        st = {"ms": round(stage_ms[n], 4)}
-        if n in flops:
-            st["tflops"] = round(flops[n] / (stage_ms[n] * 1e-3) / 1e12, 1)
-        if n in bytes_:
-            st["algorithmic_gbs"] = round(bytes_[n] / (stage_ms[n] * 1e-3) / 1e9, 1)
-        stages[n] = st
-    # ---- parity, stage by stage, each against the oracle fed with the GPU's output of the stage before
-    logits_ref = MR.matmul_ref(x16.cpu(), wg.cpu(), bg.cpu())
-    logits_ok = bool(torch.allclose(logits.cpu().float(), logits_ref.float(), rtol=2e-2, atol=2e-1))
-    ref = RR.routing_ref(logits.cpu(), k)
-    routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(r.col_sum.cpu(), ref["col_sum"])
-                      and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]))
-    n_e = 2 if args.cpu_experts <= 0 else min(args.cpu_experts, E)
-    sizes = ref["col_sum"][:n_e]
-    n_rows = int(sizes.sum())
-    t0 = time.perf_counter()
-    y1_ref = MR.matmul_ref(x8.cpu(), w1[:n_e].cpu(), b1[:n_e].cpu(), slice_sizes=sizes, gather_indx=ref["gather_indx"][:n_rows],
-                           b_mx_scale=s1[:n_e].cpu(), fused_swiglu=(1.0, 1.0))
-    y2_ref = MR.matmul_ref(y1[:n_rows].cpu(), w2[:n_e].cpu(), b2[:n_e].cpu(), slice_sizes=sizes, b_mx_scale=s2[:n_e].cpu())
-    cpu_s = time.perf_counter() - t0
-    # fp8 outputs: one step of the type (2^-3 relative) where an fp32 sum lands on a rounding boundary
-    fc1_ok = bool(torch.allclose(y1[:n_rows].cpu().float(), y1_ref.float(), rtol=0.13, atol=2e-2))
-    got2 = y2.cpu()[ref["scatter_indx"][:n_rows].long()].float()
-    # NaN marks an overflowed float8_e4m3fn output: the pattern of NaNs must agree, everything else within one step
-    ref2 = y2_ref.float()
-    nan_frac = float(torch.isnan(ref2).float().mean())
-    fc2_ok = bool(torch.equal(torch.isnan(got2), torch.isnan(ref2)) and
-                  torch.allclose(torch.nan_to_num(got2, nan=0.0), torch.nan_to_num(ref2, nan=0.0), rtol=0.13, atol=2e-2))
-    z_ref, _, _ = MR.reduce_general_ref(y2.view(T, k, d1)[:256].cpu(), 1)
-    a, b = z[:256].cpu().float(), z_ref.float()
-    combine_ok = bool(torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a), torch.nan_to_num(b)))
-    mm_ms = stage_ms["fc1_swiglu"] + stage_ms["fc2_scatter"]
-    mm_flops = flops["fc1_swiglu"] + flops["fc2_scatter"]
-    tflops = mm_flops / (mm_ms * 1e-3) / 1e12
-    out = base_line(args, "moe_mlp_tokens_per_s", round(T / (ms_per_step * 1e-3), 1), "tokens/s", ms_per_step,
+        def step(ev=None):
+            mark = (lambda i: ev[i].record()) if ev is not None else (lambda i: None)
+            mark(0)
+            logits = matmul(x16, wg, bg)
+            mark(1)
+            r = routing(logits, k)
+            mark(2)
+            y1 = matmul(x8, w1q, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
+            mark(3)
+            y2 = matmul(y1, w2q, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
+            mark(4)
+            z, _ = reduce(y2.view(T, k, d1), dim=1)
+            mark(5)
+            return logits, r, y1, y2, z
+
+        spin_up(step)
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            logits, r, y1, y2, z = step(events[i])
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        stage_ms = {n: median([e[i].elapsed_time(e[i + 1]) for e in events]) for i, n in enumerate(names)}
+        rows = T * k
+        flops = {"gate_matmul": 2.0 * T * d1 * E, "fc1_swiglu": 2.0 * rows * d1 * d2, "fc2_scatter": 2.0 * rows * (d2 // 2) * d1}
+        n_active = int((r.col_sum > 0).sum())
+        w_bytes = lambda K, N: n_active * (K // 2 * N + K // 32 * N + N * 4)
+        bytes_ = {"gate_matmul": T * d1 * 2 + d1 * E * 2 + T * E * 2, "fc1_swiglu": rows * d1 + w_bytes(d1, d2) + rows * d2 // 2,
+                  "fc2_scatter": rows * d2 // 2 + w_bytes(d2 // 2, d1) + rows * d1, "combine": rows * d1 + T * d1}
+        stages = {}
+        for n in names:
+            st = {"ms": round(stage_ms[n], 4)}
+            if n in flops:
+                st["tflops"] = round(flops[n] / (stage_ms[n] * 1e-3) / 1e12, 1)
+            if n in bytes_:
+                st["algorithmic_gbs"] = round(bytes_[n] / (stage_ms[n] * 1e-3) / 1e9, 1)
+                st["frac_of_hbm"] = round(bytes_[n] / (stage_ms[n] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+            stages[n] = st
+        # ---- parity, stage by stage, each against the oracle fed with the GPU's output of the stage before
+        logits_ref = MR.matmul_ref(x16.cpu(), wg.cpu(), bg.cpu())
+        logits_ok = bool(torch.allclose(logits.cpu().float(), logits_ref.float(), rtol=2e-2, atol=2e-1))
+        ref = RR.routing_ref(logits.cpu(), k)
+        routing_ok = bool(torch.equal(r.scatter_indx.cpu(), ref["scatter_indx"]) and torch.equal(r.col_sum.cpu(), ref["col_sum"])
+                          and torch.equal(r.gather_indx.cpu(), ref["gather_indx"]))
+        n_e = 2 if args.cpu_experts <= 0 else min(args.cpu_experts, E)
+        busy = torch.nonzero(ref["col_sum"] > 0).flatten()[:n_e].tolist()  # experts with rows (few tokens leave some empty)
+        offs = torch.cat([torch.zeros(1, dtype=torch.int64), ref["col_sum"].long().cumsum(0)])
+        fc1_ok = fc2_ok = True
+        nan_frac, n_rows, cpu_s = 0.0, 0, 0.0
+        for e in busy:
+            lo, hi = int(offs[e]), int(offs[e + 1])
+            sizes = ref["col_sum"][e:e + 1]
+            t0 = time.perf_counter()
+            y1_ref = MR.matmul_ref(x8.cpu(), w1[e:e + 1].cpu(), b1[e:e + 1].cpu(), slice_sizes=sizes,
+                                   gather_indx=ref["gather_indx"][lo:hi], b_mx_scale=s1[e:e + 1].cpu(), fused_swiglu=(1.0, 1.0))
+            y2_ref = MR.matmul_ref(y1[lo:hi].cpu(), w2[e:e + 1].cpu(), b2[e:e + 1].cpu(), slice_sizes=sizes,
+                                   b_mx_scale=s2[e:e + 1].cpu())
+            cpu_s += time.perf_counter() - t0
+            n_rows += hi - lo
+            # fp8 outputs: one step of the type (2^-3 relative) where an fp32 sum lands on a rounding boundary
+            fc1_ok = fc1_ok and bool(torch.allclose(y1[lo:hi].cpu().float(), y1_ref.float(), rtol=0.13, atol=2e-2))
+            got2 = y2.cpu()[ref["scatter_indx"][lo:hi].long()].float()
+            # NaN marks an overflowed float8_e4m3fn output: the pattern of NaNs must agree, everything else within one step
+            ref2 = y2_ref.float()
+            nan_frac += float(torch.isnan(ref2).float().sum())
+            fc2_ok = fc2_ok and bool(torch.equal(torch.isnan(got2), torch.isnan(ref2)) and
+                                     torch.allclose(torch.nan_to_num(got2, nan=0.0), torch.nan_to_num(ref2, nan=0.0), rtol=0.13, atol=2e-2))
+        nan_frac /= max(1, n_rows * d1)
+        n_chk = min(256, T)
+        z_ref, _, _ = MR.reduce_general_ref(y2.view(T, k, d1)[:n_chk].cpu(), 1)
+        a, b = z[:n_chk].cpu().float(), z_ref.float()
+        combine_ok = bool(torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a), torch.nan_to_num(b)))
+        mm_ms = stage_ms["fc1_swiglu"] + stage_ms["fc2_scatter"]
+        mm_flops = flops["fc1_swiglu"] + flops["fc2_scatter"]
+        mm_bytes = bytes_["fc1_swiglu"] + bytes_["fc2_scatter"]
+        return dict(bpe=bpe, tokens=T, rows=rows, active_experts=n_active, ms_per_step=round(ms_per_step, 4), stages=stages,
+                    mm_ms=mm_ms, mm_flops=mm_flops, mm_bytes=mm_bytes,
+                    cpu=dict(flops=2.0 * n_rows * d1 * d2 + 2.0 * n_rows * (d2 // 2) * d1, seconds=cpu_s, experts=len(busy), rows=n_rows),
+                    parity={"gate_logits_within_2e-2": logits_ok, "routing_bit_exact": routing_ok,
+                            "fc1_sample_within_fp8_step": fc1_ok, "fc2_sample_within_fp8_step": fc2_ok,
+                            "fc2_sample_overflowed_fraction": round(nan_frac, 5), "combine_bit_exact": combine_ok})
+
+    pts = [point(b) for b in bpes]
+    last = pts[-1]
+    T = last["tokens"]
+    # few rows per expert: both products stream the weights of the active experts once -- bound by HBM; at 64 rows per
+    # expert the matrix cores' share is about a third of that time
+    gbs = last["mm_bytes"] / (last["mm_ms"] * 1e-3) / 1e9
+    tflops = last["mm_flops"] / (last["mm_ms"] * 1e-3) / 1e12
+    out = base_line(args, "moe_mlp_tokens_per_s", round(T / (last["ms_per_step"] * 1e-3), 1), "tokens/s", last["ms_per_step"],
                     "fp8e4m3 x mxfp4 (fp32 accumulate), bf16 gate",
-                    f"{name}: gate matmul + routing + FC1/SwiGLU + FC2 + combine, tokens={T}, d_model={d1}, experts={E}, "
-                    f"top-{k}, W1 mxfp4 [{E},{d1},{d2}], W2 mxfp4 [{E},{d2 // 2},{d1}]", scale_layout=args.scale_layout,
-                    value_layout=args.value_layout)
-    out["stages"] = stages
-    out["roofline"] = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                       "frac": round(tflops / PEAK_FP8_TFLOPS, 4), "traffic": None, "kernel": "mm_x8_mxfp4_kernel (FC1 + FC2)",
-                       "kernel_ms": round(mm_ms, 4), "algorithmic_flops": mm_flops,
-                       "algorithmic_bytes": bytes_["fc1_swiglu"] + bytes_["fc2_scatter"],
-                       "hbm_gbs": round((bytes_["fc1_swiglu"] + bytes_["fc2_scatter"]) / (mm_ms * 1e-3) / 1e9, 1)}
-    out["cpu_baseline"] = {"value": round((2.0 * n_rows * d1 * d2 + 2.0 * n_rows * (d2 // 2) * d1) / cpu_s / 1e12, 5),
-                           "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
-                           "sample": f"oracle FC1 + FC2 on the first {n_e} of {E} experts ({n_rows} of {rows} rows), {cpu_s:.1f} s"}
-    out["parity"] = {"gate_logits_within_2e-2": logits_ok, "routing_bit_exact": routing_ok, "fc1_sample_within_fp8_step": fc1_ok,
-                     "fc2_sample_within_fp8_step": fc2_ok, "fc2_sample_overflowed_fraction": round(nan_frac, 5),
-                     "combine_bit_exact": combine_ok}
+                    f"{name}: gate matmul + routing + FC1/SwiGLU + FC2 + combine, tokens={T} ({last['bpe']} rows per expert), "
+                    f"d_model={d1}, experts={E}, top-{k}, W1 mxfp4 [{E},{d1},{d2}], W2 mxfp4 [{E},{d2 // 2},{d1}]",
+                    scale_layout=args.scale_layout, value_layout=args.value_layout)
+    out["stages"] = last["stages"]
+    out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_x8_mxfp4_kernel (FC1 + FC2)",
+                       "kernel_ms": round(last["mm_ms"], 4), "algorithmic_flops": last["mm_flops"],
+                       "algorithmic_bytes": last["mm_bytes"], "tflops": round(tflops, 1),
+                       "frac_of_fp8_mfma_peak": round(tflops / PEAK_FP8_TFLOPS, 4)}
+    c = last["cpu"]
+    out["cpu_baseline"] = {"value": round(c["flops"] / max(c["seconds"], 1e-9) / 1e12, 5), "unit": "TFLOP/s",
+                           "cores": os.cpu_count(), "kind": "port",
+                           "sample": f"oracle FC1 + FC2 on {c['experts']} of {E} experts ({c['rows']} of {last['rows']} rows), {c['seconds']:.1f} s"}
+    out["parity"] = last["parity"]
+    if len(pts) > 1:
+        out["sweep"] = [{"bpe": p["bpe"], "tokens": p["tokens"], "active_experts": p["active_experts"], "ms_per_step": p["ms_per_step"],
+                         "stages": p["stages"], "parity_all_true": all(v is True for k_, v in p["parity"].items() if isinstance(v, bool))}
+                        for p in pts]
     return out
 
 
@@ -768,6 +802,7 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: leave out the short runs of the other configurations")
     ap.add_argument("--block-m", type=int, default=0)
+    ap.add_argument("--bpe", type=int, default=0, help="--workload mlp: rows per expert (tokens = bpe * experts / top-k)")
     ap.add_argument("--scale-layout", default=None, choices=["strided", "cdna4"],
                     help="encoding of the weight scales handed to matmul: [E, K/32, N] bytes contiguous along K, or the "
                     "CDNA4 pre-shuffle (convert_layout(..., CDNA4MXScaleLayout())).  Default: cdna4, what the reference "
