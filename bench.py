@@ -11,6 +11,7 @@ product, routing, decode, fp8 down projection + combine, quantise, dequantise), 
 achieved rate, roofline fraction and parity flags.
 """
 import argparse
+import gc
 import hashlib
 import json
 import os
@@ -119,6 +120,20 @@ def median(xs):
     return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
 
 
+class quiet_host:
+    """Around a timed region: the collector runs once before it and not inside it.  A collection that frees large
+    temporaries (the weights' float32 originals, layout conversions) inside the region returns their memory to the
+    driver, which waits for the GPU -- tens of milliseconds charged to a few dozen steps."""
+
+    def __enter__(self):
+        gc.collect()
+        gc.disable()
+        torch.cuda.synchronize()
+
+    def __exit__(self, *exc):
+        gc.enable()
+
+
 def timed(fn, steps, warmup):
     """Runs fn warmup + steps times for the wall time per call, then steps times again with a pair of HIP events around
     every call for the kernel time: for calls of a few tens of microseconds the event records themselves (host time and
@@ -128,12 +143,12 @@ def timed(fn, steps, warmup):
     spin_up(fn)
     for _ in range(warmup):
         out = fn()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        out = fn()
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
+    with quiet_host():
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = fn()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for a, b in ev:
         a.record()
@@ -415,12 +430,12 @@ def run_fc2(args, cfg, name):
             r, gam, y, z = step()
         torch.cuda.synchronize()
         events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            r, gam, y, z = step(events[i])
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+        with quiet_host():
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                r, gam, y, z = step(events[i])
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = median([e[0].elapsed_time(e[1]) for e in events])
     combine_ms = median([e[2].elapsed_time(e[3]) for e in events])
@@ -530,12 +545,12 @@ def run_fc1(args, cfg, name):
             r, y = step()
         torch.cuda.synchronize()
         events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            r, y = step(events[i])
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+        with quiet_host():
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                r, y = step(events[i])
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = median([a.elapsed_time(b) for a, b in events])
 
@@ -639,6 +654,8 @@ def run_mlp(args, cfg, name):
     pc2 = PrecisionConfig(b_mx_scale=scales_for_matmul(s2, args.scale_layout), b_microblock_size=32)
     act1 = FusedActivation(FnSpecs("swiglu", swiglu_fn, ("alpha", "limit"), reduction_n=2), (1.0, 1.0))
     names = ("gate_matmul", "routing", "fc1_swiglu", "fc2_scatter", "combine")
+    from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
+    constraints = {"block_m": args.block_m} if args.block_m else {}
 
     def point(bpe):
         T = bpe * E // k
@@ -652,9 +669,10 @@ def run_mlp(args, cfg, name):
             mark(1)
             r = routing(logits, k)
             mark(2)
-            y1 = matmul(x8, w1q, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
-            mark(3)
-            y2 = matmul(y1, w2q, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
+            with scoped_opt_flags_constraints(constraints):
+                y1 = matmul(x8, w1q, b1, r.ragged_metadata, gather_indx=r.gather_indx, precision_config=pc1, fused_activation=act1)
+                mark(3)
+                y2 = matmul(y1, w2q, b2, r.ragged_metadata, scatter_indx=r.scatter_indx, precision_config=pc2)
             mark(4)
             z, _ = reduce(y2.view(T, k, d1), dim=1)
             mark(5)
@@ -665,11 +683,12 @@ def run_mlp(args, cfg, name):
             step()
         torch.cuda.synchronize()
         events = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            logits, r, y1, y2, z = step(events[i])
-        torch.cuda.synchronize()
-        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        with quiet_host():
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                logits, r, y1, y2, z = step(events[i])
+            torch.cuda.synchronize()
+            ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
         stage_ms = {n: median([e[i].elapsed_time(e[i + 1]) for e in events]) for i, n in enumerate(names)}
         rows = T * k
         flops = {"gate_matmul": 2.0 * T * d1 * E, "fc1_swiglu": 2.0 * rows * d1 * d2, "fc2_scatter": 2.0 * rows * (d2 // 2) * d1}

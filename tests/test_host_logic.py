@@ -78,6 +78,12 @@ def test_opt_flags_constraints_scope_and_errors():
     assert OF.make_opt_flags(256, 5760, 2880, 128, True).block_m == 16
     assert OF.make_opt_flags(256, 4096, 2048, 1, False).block_m == 128
     assert OF.make_opt_flags(1000, 64, 64, 10, True, expected_slice_size=40).block_m == 64
+    # the block covers the mean slice and two standard deviations of a Poisson-like size: 16 + 8 -> 32, 64 + 16 -> 128,
+    # 2 + 2.8 -> 16 (decode); fp8 rows never take the 16-row block (the streaming kernel would widen them to 16 bits)
+    assert OF.make_opt_flags(2048, 5760, 2880, 128, True).block_m == 32
+    assert OF.make_opt_flags(8192, 5760, 2880, 128, True).block_m == 128
+    assert OF.make_opt_flags(256, 5760, 2880, 128, True, fp8_rows=True).block_m == 32
+    assert OF.make_opt_flags(256, 5760, 2880, 1, False, fp8_rows=True).block_m == 128  # dense: rows as they are
     with OF.scoped_opt_flags_constraints({"block_m": 32}):
         assert OF.make_opt_flags(16384, 5760, 2880, 128, True).block_m == 32
         with OF.scoped_opt_flags_constraints({"block_m": 64}):

@@ -279,7 +279,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         raise NotImplementedError(f"fused activation {fused_activation.specs.name!r} is not built")
     # ---- tile choice
     flags = make_opt_flags(M, N, K, n_slices, ragged,
-                           a_ragged_metadata.expected_slice_size if ragged else None)
+                           a_ragged_metadata.expected_slice_size if ragged else None,
+                           fp8_rows=a.dtype in fp8_types and b_fp4)
     args = _lib.MatmulArgBag()
     args.x, args.x_dtype = a.data_ptr(), _lib.dtype_code(a.dtype)
     args.x_stride_m = a.stride(-2)

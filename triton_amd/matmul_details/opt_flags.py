@@ -83,10 +83,13 @@ def max_allowable_mn(max_mn: int, m: int, n: int, split_k: int) -> int:
 
 
 def make_opt_flags(m: int, n: int, k: int, n_slices: int, ragged: bool,
-                   expected_slice_size: Optional[int] = None) -> OptFlags:
-    """Picks BLOCK_M from the expected rows per slice (no device read): the smallest
-    tile that covers them, capped at 128, so that ragged slices waste at most one
-    partly filled 16-row fragment per block.
+                   expected_slice_size: Optional[int] = None, fp8_rows: bool = False) -> OptFlags:
+    """Picks BLOCK_M from the expected rows per slice (no device read): the smallest tile, capped at 128, that covers
+    the mean and two standard deviations of a slice's size (the sizes of routed slices scatter about like a Poisson
+    count), so that nearly every slice is ONE row block: a second block streams the slice's weights a second time,
+    which at 16 to 64 rows per slice costs 10 to 40 % (measured on the layer of the reference's bench_mlp).  Row
+    blocks of 16 run the weight-streaming kernel, which expands fp8 rows to 16 bits; fp8 rows are faster through the
+    tiled kernel's scaled MFMA, whose smallest useful block is 32 (`fp8_rows`).
 
     Constraints are validated as the reference validates them (opt_flags.py:71-73, 46-50): an unknown key is
     an AssertionError; a known key has to hold for the flags that come out, and since the tile's width, depth
@@ -115,7 +118,10 @@ def make_opt_flags(m: int, n: int, k: int, n_slices: int, ragged: bool,
     rows = m
     if ragged:
         rows = expected_slice_size if expected_slice_size is not None else max(1, m // max(1, n_slices))
-    block_m = next((b for b in BLOCK_M_CHOICES if rows <= b), BLOCK_M_CHOICES[-1])
+    cover = rows + 2.0 * rows ** 0.5 if ragged else rows
+    block_m = next((b for b in BLOCK_M_CHOICES if cover <= b), BLOCK_M_CHOICES[-1])
+    if ragged and fp8_rows and block_m == 16:
+        block_m = 32
     if c.get("block_m") is not None:
         block_m = int(c["block_m"])
         if block_m not in BLOCK_M_CHOICES:
