@@ -40,6 +40,7 @@ WORKLOADS = {
     # fc1_prefill with the activations quantised to MXFP8 inside the step (downcast_to_mxfp + scaled-MFMA matmul):
     # the block-scaled fp8 x fp4 path of the hardware; NOT interchangeable with the bf16 workload (x loses precision)
     "fc1_prefill_mx8": dict(T=4096, E=128, k=4, K=2880, N=5760, act=True, mx8=True),
+    "fc1_prefill_mx4": dict(T=4096, E=128, k=4, K=2880, N=5760, act=True, mx4=True),
     # the down projection at decode size (fp8 rows of 64 tokens): weight streaming through the tiled fp8 kernel
     "fc2_decode": dict(T=64, E=128, k=4, K=2880, N=2880, act=False, fc2=True),
     # BASELINE config 1: one dense bf16 x MXFP4 product with bias (launch / latency bound: 7.6 MB, 4.3 GFLOP)
@@ -341,13 +342,14 @@ def run_quant(args, cfg, name):
     return out
 
 
-def algorithmic_bytes(col_sum, T, k, K, N, act):
-    """x rows read + y rows written + (codes + scales + bias) of the experts that have rows."""
+def algorithmic_bytes(col_sum, T, k, K, N, act, x_row_bytes=None):
+    """x rows read + y rows written + (codes + scales + bias) of the experts that have rows.  `x_row_bytes`: one
+    activation row as stored (bf16 unless given: MXFP8 K + K/32, MXFP4 K/2 + K/32)."""
     rows = T * k
     n_active = int((col_sum > 0).sum())
     n_out = N // 2 if act else N
     per_expert = K // 2 * N + K // 32 * N + N * 2
-    return rows * K * 2 + rows * n_out * 2 + n_active * per_expert, n_active
+    return rows * (x_row_bytes or K * 2) + rows * n_out * 2 + n_active * per_expert, n_active
 
 
 def cpu_baseline(x_cpu, vals, scales, bias_cpu, ref, experts, K, N, act, fc2=None):
@@ -520,14 +522,16 @@ def run_fc1(args, cfg, name):
     constraints = {"block_m": args.block_m} if args.block_m else {}
     wq = weights_for_matmul(vals, args.value_layout)
 
-    mx8 = bool(cfg.get("mx8"))
+    mx4 = bool(cfg.get("mx4"))   # MXFP4 activations: packed e2m1 codes, widened (exactly) to fp8 inside matmul
+    mx8 = bool(cfg.get("mx8")) or mx4
+    x_store = torch.uint8 if mx4 else torch.float8_e4m3fn
     if mx8:
         from triton_amd.numerics_details.mxfp import downcast_to_mxfp
 
     def step(ev=None):
         r = routing(logits, k)
         if mx8:
-            xq, xs = downcast_to_mxfp(x, torch.float8_e4m3fn, axis=-1)
+            xq, xs = downcast_to_mxfp(x, x_store, axis=-1)
             pcs = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=pc.b_mx_scale, b_microblock_size=32)
         if ev is not None:
             ev[0].record()
@@ -557,11 +561,14 @@ def run_fc1(args, cfg, name):
     col_sum = r.col_sum.cpu()
     rows = T * k
     flops = 2.0 * rows * K * N
-    abytes, n_active = algorithmic_bytes(col_sum, T, k, K, N, act)
+    x_row_bytes = (K // 2 if mx4 else K) + K // 32 if mx8 else None
+    abytes, n_active = algorithmic_bytes(col_sum, T, k, K, N, act, x_row_bytes)
     tflops_step = flops / (ms_per_step * 1e-3) / 1e12
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
     gbs_kernel = abytes / (kernel_ms * 1e-3) / 1e9
-    peak_mfma = PEAK_FP8_TFLOPS if mx8 else PEAK_BF16_TFLOPS
+    # the operands' own peak decides which roofline binds (MXFP4 x MXFP4: 10.1 PFLOP/s, so the bytes bind); the
+    # kernel multiplies widened fp8 values either way
+    peak_mfma = PEAK_MXFP4_TFLOPS if mx4 else PEAK_FP8_TFLOPS if mx8 else PEAK_BF16_TFLOPS
     hbm_bound = (abytes / (PEAK_HBM_GBS * 1e9)) > (flops / (peak_mfma * 1e12))
     traffic, traffic_source = measured_traffic(name)
     if hbm_bound:
@@ -572,6 +579,9 @@ def run_fc1(args, cfg, name):
                     frac=round(tflops_kernel / peak_mfma, 4), traffic=traffic, traffic_source=traffic_source)
     # row blocks of 16 (few rows per expert) run the weight-streaming kernel, everything else the tiled one
     roof["kernel"] = "mm_stream16_kernel" if rows <= 16 * E else ("mm_x8_mxfp4_kernel" if mx8 else "mm_x16_mxfp4_kernel")
+    if mx4:
+        roof["kernel"] = "widen_e2m1_rows_kernel + " + roof["kernel"]
+        roof["frac_of_fp8_mfma_peak"] = round(tflops_kernel / PEAK_FP8_TFLOPS, 4)
     roof["kernel_ms"] = round(kernel_ms, 4)
     roof["algorithmic_bytes"] = abytes
     roof["algorithmic_flops"] = flops
@@ -595,7 +605,7 @@ def run_fc1(args, cfg, name):
         x_ref = x_cpu
         if mx8:  # the oracle sees the same quantised activations, dequantised (exactly) to bf16
             from oracle.mxfp_ref import downcast_to_mxfp_ref, upcast_from_mxfp_ref
-            qv, qs = downcast_to_mxfp_ref(x_cpu, torch.float8_e4m3fn, axis=-1)
+            qv, qs = downcast_to_mxfp_ref(x_cpu, x_store, axis=-1)
             x_ref = upcast_from_mxfp_ref(qv, qs, torch.bfloat16, axis=-1)
         y_ref, n_rows, cpu_tflops, cpu_s = cpu_baseline(x_ref, vals, scales, bias_cpu, ref, n_e, K, N, act)
         gemm_ok = bool(torch.allclose(y[:n_rows].cpu().float(), y_ref.float(), rtol=1e-2, atol=1e-2))
@@ -603,7 +613,8 @@ def run_fc1(args, cfg, name):
                    sample=f"oracle matmul_ref (dequantise + fp32 GEMM + SwiGLU) on the first {n_e} of {E} experts "
                           f"({n_rows} of {rows} rows), {cpu_s:.1f} s")
     out = base_line(args, "moe_matmul_ogs_tflops", round(tflops_step, 2), "TFLOP/s", ms_per_step,
-                    ("mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") + " (fp32 accumulate)",
+                    ("mxfp4 x mxfp4 (multiplied as fp8)" if mx4 else "mxfp8 x mxfp4" if mx8 else "bf16 x mxfp4") +
+                    " (fp32 accumulate)",
                     f"{name}: routing + " + ("downcast_to_mxfp(x) + " if mx8 else "") +
                     f"matmul_ogs(gather, grouped GEMM, bias+SwiGLU), T={T}, hidden={K}, experts={E}, top-{k}, "
                     f"W1 mxfp4 [{E},{K},{N}]", rows=rows, active_experts=n_active, scale_layout=args.scale_layout,

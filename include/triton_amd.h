@@ -91,6 +91,15 @@ int tamd_upcast_mxfp(const void *vals, int val_dtype, int64_t val_stride_b, int6
                      int64_t dst_stride_b, int64_t dst_stride_l, int64_t dst_stride_r, void *stream);
 
 /*
+ * MXFP4 activations of the matmul (matmul.py:131-136, 772-778: a_mx_scale with e2m1 values): the reference's kernel
+ * loads the packed codes itself; here the rows are widened, exactly, to float8_e4m3fn (every e2m1 number is an e4m3
+ * number) and run through the MXFP8 path of tamd_matmul with the same e8m0 scales.
+ * src: rows x row_bytes packed bytes (two codes each, low nibble = even index), dst: rows x 2 * row_bytes bytes.
+ */
+int tamd_widen_mxfp4_rows(const uint8_t *src, int64_t rows, int64_t row_bytes, int64_t src_stride, uint8_t *dst,
+                          int64_t dst_stride, void *stream);
+
+/*
  * topk forward: replaces the launch of _topk_forward (topk.py:58-67; kernel
  * topk_details/_topk_forward.py:87-147).
  *

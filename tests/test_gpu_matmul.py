@@ -12,7 +12,8 @@ from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
 from triton_amd.numerics_details.mxfp import downcast_to_mxfp
 from triton_amd.routing import routing
 from triton_amd.swiglu import swiglu_fn
-from triton_amd.tensor import make_ragged_tensor_metadata
+from triton_amd.tensor import FP4, convert_layout, make_ragged_tensor_metadata, wrap_torch_tensor
+from triton_amd.tensor_details.layout import CDNA4MXValueLayout
 from triton_amd.testing import assert_close
 
 pytestmark = pytest.mark.gpu
@@ -683,6 +684,176 @@ def test_mxfp8_activations_ragged(block_m, cdna4_scales, device):
                      precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0), c=out_init)
     ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, a_mx_scale=rxs,
                         b_mx_scale=rs, gammas=gammas, fused_swiglu=(1.702, 7.0))
+    check(out, ref)
+
+
+# ---------------------------------------------------------------------------- MXFP4 activations
+
+
+def in_blocks(v):
+    """MXFP4 codes as downcast_to_mxfp returns them -> the kernels' block layout."""
+    return convert_layout(wrap_torch_tensor(v, dtype=FP4), CDNA4MXValueLayout())
+
+
+def quantize_x_mxfp4(x0, device):
+    """fp32 [.., K] -> (packed e2m1 codes [.., K/2], e8m0 scales per 32 along K) on the GPU, checked against the oracle."""
+    xq, xs = downcast_to_mxfp(x0.to(device), torch.uint8, axis=-1)
+    rq, rs = downcast_to_mxfp_ref(x0, torch.uint8, axis=-1)
+    assert torch.equal(xq.cpu(), rq) and torch.equal(xs.cpu(), rs)
+    return xq, xs, rq.contiguous(), rs.contiguous()
+
+
+def test_widen_mxfp4_rows_every_code(device):
+    """All 256 bytes: the widened pair of float8_e4m3fn numbers has the values of the two e2m1 codes, low nibble
+    first, with the sign of zero kept; row strides honoured."""
+    from triton_amd import _lib
+    from oracle.mxfp_ref import upcast_from_mxfp_ref
+    src = torch.arange(256, dtype=torch.uint8).reshape(4, 64)
+    wide = torch.zeros((4, 160), dtype=torch.uint8, device=device)
+    d = src.to(device)
+    rc = _lib.lib().tamd_widen_mxfp4_rows(_lib.ptr(d), 4, 64, 64, _lib.ptr(wide), 160, _lib.stream_ptr(d.device))
+    assert rc == 0
+    got = wide.cpu()
+    assert torch.all(got[:, 128:] == 0)
+    unit = torch.full((4, 4), 127, dtype=torch.uint8)                     # scale 2^0 for each 32 values
+    want = upcast_from_mxfp_ref(src, unit, torch.float32, axis=-1)
+    vals = got[:, :128].contiguous().view(torch.float8_e4m3fn).float()
+    assert torch.equal(vals, want) and torch.equal(torch.signbit(vals), torch.signbit(want))
+
+
+@pytest.mark.parametrize("swizzled", [False, True])
+def test_mxfp4_activations_mxfp4_weights_plain(swizzled, device):
+    """tests/test_matmul.py:234-235 of the reference: 256 x 256 x 256, both operands MXFP4, bf16 output."""
+    torch.manual_seed(0)
+    M = K = N = 256
+    x0 = torch.randn(M, K) * torch.exp(torch.randn(M, K // 32).repeat_interleave(32, dim=1) * 2)
+    w = torch.randn(K, N) * 0.02
+    v, s, rv, rs = quantize_w(w, device)
+    xq, xs, rq, rxs = quantize_x_mxfp4(x0, device)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=preshuffle(s) if swizzled else s,
+                         b_microblock_size=32, out_dtype=torch.bfloat16)
+    out = matmul(wrap_torch_tensor(xq, dtype=FP4), in_blocks(v) if swizzled else v, None, precision_config=pc)
+    ref = MR.matmul_ref(rq, rv, None, a_mx_scale=rxs, b_mx_scale=rs)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (M, N)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=RTOL, atol=ATOL * float(ref.float().abs().max()) / 4 + ATOL)
+    # the raw uint8 tensor is taken as packed codes too, and the product is linear in the block scales
+    pc32 = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float32)
+    pc32b = PrecisionConfig(a_mx_scale=xs + 1, a_microblock_size=32, b_mx_scale=s, b_microblock_size=32, out_dtype=torch.float32)
+    y = matmul(xq, v, None, precision_config=pc32)
+    assert torch.equal(matmul(xq, v, None, precision_config=pc32b), 2 * y)
+    # e2m1 codes widened to fp8 are the same numbers: the MXFP8 path with the widened values gives the same bits
+    from oracle.mxfp_ref import upcast_from_mxfp_ref
+    unit = torch.full_like(rxs, 127)
+    x8 = upcast_from_mxfp_ref(rq, unit, torch.float32, axis=-1).to(torch.float8_e4m3fn).to(device)
+    assert torch.equal(matmul(x8, v, None, precision_config=pc32), y)
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 64, 128])
+@pytest.mark.parametrize("cdna4", [False, True])
+def test_mxfp4_activations_mxfp4_weights_ragged(block_m, cdna4, device):
+    """Gather, scatter with dropped rows, gate weights, SwiGLU on MXFP4 x MXFP4; with `cdna4` the weights are in the
+    CDNA4 value layout and their scales in the CDNA4 scale layout."""
+    torch.manual_seed(1)
+    E, K, N = 7, 320, 400 if not cdna4 else 448
+    sizes = torch.tensor([3, 0, 1, 16, 5, 140, 2], dtype=torch.int32)
+    M = int(sizes.sum())
+    x0 = torch.randn(M + 5, K) * torch.exp(torch.randn(M + 5, K // 32).repeat_interleave(32, dim=1))
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    xq, xs, rq, rxs = quantize_x_mxfp4(x0, device)
+    gather = torch.randint(0, M + 5, (M, ), dtype=torch.int32)
+    scatter = torch.randperm(M, dtype=torch.int32)
+    scatter[::7] = -1
+    gammas = 2.0**torch.randint(-3, 1, (M, )).float()
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=preshuffle(s) if cdna4 else s,
+                         b_microblock_size=32)
+    out_init = torch.zeros((M, N // 2), dtype=torch.bfloat16, device=device)
+    with scoped_opt_flags_constraints({} if block_m is None else {"block_m": block_m}):
+        out = matmul(xq, in_blocks(v) if cdna4 else v, bias.to(device), md, gather_indx=gather.to(device),
+                     scatter_indx=scatter.to(device), precision_config=pc, gammas=gammas.to(device),
+                     fused_activation=swiglu_act(1.702, 7.0), c=out_init)
+    ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, a_mx_scale=rxs,
+                        b_mx_scale=rs, gammas=gammas, fused_swiglu=(1.702, 7.0))
+    check(out, ref)
+
+
+def test_mxfp4_activations_prefill_shape(device):
+    """The shape of the prefill up projection (K 2880, N 5760, 4 of 128 experts with rows; 1 row to several row
+    blocks), MXFP4 activations against MXFP4 weights in the CDNA4 layouts."""
+    torch.manual_seed(2)
+    E, K, N = 6, 2880, 5760
+    sizes = torch.tensor([300, 0, 1, 129, 64, 0], dtype=torch.int32)
+    M = int(sizes.sum())
+    x0 = torch.randn(M, K) * torch.exp(torch.randn(M, K // 32).repeat_interleave(32, dim=1))
+    w = torch.randn(E, K, N) * 0.02
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    xq, xs, rq, rxs = quantize_x_mxfp4(x0, device)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=preshuffle(s), b_microblock_size=32)
+    out = matmul(xq, in_blocks(v), bias.to(device), md, precision_config=pc, fused_activation=swiglu_act(1.702, 7.0))
+    ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, a_mx_scale=rxs, b_mx_scale=rs, fused_swiglu=(1.702, 7.0))
+    check(out, ref)
+
+
+@pytest.mark.parametrize("mode", ["ragged", "batched"])
+@pytest.mark.parametrize("w_dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("a_kind", ["mxfp4", "mxfp8"])
+def test_mx_activations_16bit_weights(mode, w_dtype, a_kind, device):
+    """tests/test_matmul.py:217-232 of the reference: 64 x 128 x 96, microscaled activations against unquantised
+    bf16 / fp16 weights, bf16 output."""
+    torch.manual_seed(3)
+    M, N, K = 64, 128, 96
+    E = 3
+    quant = quantize_x_mxfp4 if a_kind == "mxfp4" else quantize_x_mxfp8
+    if mode == "ragged":
+        sizes = torch.tensor([20, 0, 44], dtype=torch.int32)
+        x0 = torch.randn(M, K) * torch.exp(torch.randn(M, K // 32).repeat_interleave(32, dim=1))
+    else:
+        x0 = torch.randn(E, M, K) * torch.exp(torch.randn(E, M, K // 32).repeat_interleave(32, dim=2))
+    w = (torch.randn(E, K, N) * 0.1).to(w_dtype)
+    bias = torch.randn(E, N)
+    xq, xs, rq, rxs = quant(x0, device)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, out_dtype=torch.bfloat16)
+    if mode == "ragged":
+        md = make_ragged_tensor_metadata(sizes.to(device), M)
+        out = matmul(xq, w.to(device), bias.to(device), md, precision_config=pc)
+        ref = MR.matmul_ref(rq, w, bias, slice_sizes=sizes, a_mx_scale=rxs)
+    else:
+        out = matmul(xq, w.to(device), bias.to(device), precision_config=pc)
+        ref = MR.matmul_ref(rq, w, bias, a_mx_scale=rxs)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == tuple(ref.shape)
+    check(out, ref)
+
+
+@pytest.mark.parametrize("mode", ["ragged", "batched"])
+def test_mxfp8_activations_mxfp8_weights(mode, device):
+    """tests/test_matmul.py:214-216 of the reference: 300 x 400 x 416, both operands MXFP8."""
+    torch.manual_seed(4)
+    M, N, K = 300, 400, 416
+    E = 3
+    if mode == "ragged":
+        sizes = torch.tensor([120, 0, 180], dtype=torch.int32)
+        x0 = torch.randn(M, K) * torch.exp(torch.randn(M, K // 32).repeat_interleave(32, dim=1))
+    else:
+        x0 = torch.randn(E, M, K) * torch.exp(torch.randn(E, M, K // 32).repeat_interleave(32, dim=2))
+    w = torch.randn(E, K, N) * 0.05
+    bias = torch.randn(E, N)
+    wq, ws = downcast_to_mxfp(w.to(device), torch.float8_e4m3fn, axis=-2)
+    rwq, rws = downcast_to_mxfp_ref(w, torch.float8_e4m3fn, axis=-2)
+    assert torch.equal(wq.cpu().view(torch.uint8), rwq.contiguous().view(torch.uint8)) and torch.equal(ws.cpu(), rws)
+    xq, xs, rq, rxs = quantize_x_mxfp8(x0, device)
+    pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=ws, b_microblock_size=32,
+                         out_dtype=torch.bfloat16)
+    if mode == "ragged":
+        md = make_ragged_tensor_metadata(sizes.to(device), M)
+        out = matmul(xq, wq, bias.to(device), md, precision_config=pc)
+        ref = MR.matmul_ref(rq, rwq, bias, slice_sizes=sizes, a_mx_scale=rxs, b_mx_scale=rws)
+    else:
+        out = matmul(xq, wq, bias.to(device), precision_config=pc)
+        ref = MR.matmul_ref(rq, rwq, bias, a_mx_scale=rxs, b_mx_scale=rws)
     check(out, ref)
 
 

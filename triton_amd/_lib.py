@@ -110,6 +110,7 @@ _SIGNATURES = {
                             _INT, _PTR], C.c_int),
     "tamd_upcast_mxfp": ([_PTR, _INT, _I64, _I64, _PTR, _I64, _I64, _PTR, _INT, _I64, _I64, _I64, _I64, _I64, _I64,
                           _PTR], C.c_int),
+    "tamd_widen_mxfp4_rows": ([_PTR, _I64, _I64, _I64, _PTR, _I64, _PTR], C.c_int),
     "tamd_topk_forward": ([_PTR, _INT, _I64, _INT, _INT, _INT, _INT, _INT, _PTR, _PTR, _I64, _PTR, _I64, _I64, _PTR],
                           C.c_int),
     "tamd_bitmatrix_metadata_workspace": ([_I64, _INT], C.c_int64),

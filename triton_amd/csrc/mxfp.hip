@@ -623,9 +623,63 @@ int launch_upcast(const uint8_t *vals, int64_t vsb, int64_t vsr, const uint8_t *
   return launch_status();
 }
 
+// e2m1 codes -> float8_e4m3fn bytes, exactly: every e2m1 number (0, .5, 1, 1.5, 2, 3, 4, 6 and their negatives) is an
+// e4m3 number.  A thread widens 16 packed bytes (32 codes, low nibble first) of a row to 32 bytes.
+__global__ __launch_bounds__(256) void widen_e2m1_rows_kernel(const uint8_t *__restrict__ src, int64_t rows, int64_t row_bytes,
+                                                              int64_t src_stride, uint8_t *__restrict__ dst, int64_t dst_stride,
+                                                              int vec) {
+  // magnitudes 0..7 as e4m3 bytes, one table entry per byte of two 32-bit words
+  constexpr uint32_t kLo = 0x3C383000u, kHi = 0x4C484440u;  // {0x00, 0x30, 0x38, 0x3C}, {0x40, 0x44, 0x48, 0x4C}
+  auto widen = [&](uint32_t code) -> uint32_t {              // one nibble -> one byte
+    const uint32_t mag = code & 7u;
+    const uint32_t tab = mag < 4u ? kLo : kHi;
+    return ((tab >> (8 * (mag & 3u))) & 0xFFu) | ((code & 8u) << 4);
+  };
+  auto widen4 = [&](uint32_t two_bytes) -> uint32_t {        // four nibbles (16 bits) -> four bytes
+    return widen(two_bytes) | (widen(two_bytes >> 4) << 8) | (widen(two_bytes >> 8) << 16) | (widen(two_bytes >> 12) << 24);
+  };
+  const int64_t chunks = (row_bytes + 15) / 16, total = rows * chunks;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / chunks, c = (i - r * chunks) * 16;
+    const uint8_t *sp = src + r * src_stride + c;
+    uint8_t *dp = dst + r * dst_stride + 2 * c;
+    if (vec && c + 16 <= row_bytes) {
+      const uint4 q = *(const uint4 *)sp;
+      const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+      uint32_t o[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        o[2 * j] = widen4(w[j] & 0xFFFFu);
+        o[2 * j + 1] = widen4(w[j] >> 16);
+      }
+      *(uint4 *)dp = make_uint4(o[0], o[1], o[2], o[3]);
+      *(uint4 *)(dp + 16) = make_uint4(o[4], o[5], o[6], o[7]);
+    } else {
+      for (int64_t b = 0; b < 16 && c + b < row_bytes; ++b) {
+        const uint32_t v = sp[b];
+        dp[2 * b] = (uint8_t)widen(v);
+        dp[2 * b + 1] = (uint8_t)widen(v >> 4);
+      }
+    }
+  }
+}
+
 }  // namespace tamd
 
 using namespace tamd;
+
+extern "C" int tamd_widen_mxfp4_rows(const uint8_t *src, int64_t rows, int64_t row_bytes, int64_t src_stride, uint8_t *dst,
+                                     int64_t dst_stride, void *stream) {
+  if (rows < 0 || row_bytes < 0) return TAMD_E_INVALID;
+  if (rows == 0 || row_bytes == 0) return 0;
+  if (!src || !dst) return TAMD_E_INVALID;
+  const int vec = aligned(src, 16) && aligned(dst, 16) && src_stride % 16 == 0 && dst_stride % 16 == 0;
+  int64_t blocks = (rows * ((row_bytes + 15) / 16) + 255) / 256;
+  blocks = blocks > 65536 * 16 ? 65536 * 16 : blocks;
+  widen_e2m1_rows_kernel<<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(src, rows, row_bytes, src_stride, dst,
+                                                                                 dst_stride, vec);
+  return launch_status();
+}
 
 extern "C" int tamd_downcast_mxfp(const void *src, int src_dtype, int64_t nb, int64_t L, int64_t nr,
                                   int64_t src_stride_b, int64_t src_stride_l, int64_t src_stride_r,

@@ -81,6 +81,21 @@ def _data(t):
     return t.storage.data if isinstance(t, Tensor) else t
 
 
+def _widen_mxfp4_activations(a_raw):
+    """MXFP4 activations (packed e2m1 codes along K with one e8m0 byte per 32, matmul.py:131-136 of the reference)
+    against MXFP4 weights: the codes are widened -- exactly: every e2m1 number is a float8_e4m3fn number -- and take
+    the MXFP8 path of the kernels with the same scales."""
+    _lib.require_gpu(a_raw, "a")
+    assert a_raw.stride(-1) == 1, "packed activations must be contiguous along K"
+    rows = a_raw.numel() // a_raw.shape[-1]
+    src = a_raw if a_raw.is_contiguous() else a_raw.contiguous()
+    out = torch.empty((*a_raw.shape[:-1], 2 * a_raw.shape[-1]), dtype=torch.float8_e4m3fn, device=a_raw.device)
+    rc = _lib.lib().tamd_widen_mxfp4_rows(_lib.ptr(src), rows, src.shape[-1], src.shape[-1], _lib.ptr(out),
+                                          out.shape[-1], _lib.stream_ptr(a_raw.device))
+    _lib.check(rc, "matmul (MXFP4 activations)")
+    return out
+
+
 _TURNED = {}  # id(weights) -> (weak reference to them, their version counter, the copy with unit stride along K)
 
 
@@ -155,10 +170,25 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
     if a_mx_scale is not None:
         a_mx_scale = _data(a_mx_scale)
         a_raw = a.storage.data if isinstance(a, Tensor) else a
-        if a_raw.dtype != torch.float8_e4m3fn or a_mx_scale.dtype != torch.uint8:
-            raise NotImplementedError("microscaled activations are built for float8_e4m3fn values with e8m0 scales")
+        a_fp4 = a_raw.dtype == torch.uint8 and (not isinstance(a, Tensor) or a.dtype == FP4)
+        if not (a_fp4 or a_raw.dtype == torch.float8_e4m3fn) or a_mx_scale.dtype != torch.uint8:
+            raise NotImplementedError("microscaled activations are built for float8_e4m3fn or packed e2m1 values "
+                                      "with e8m0 scales")
         mb = precision_config.a_microblock_size
         assert mb is None or mb == MXFP_BLOCK_SIZE, "Unsupported microscale block size"
+        b_raw = _data(b)
+        b_packed = b.dtype == FP4 if isinstance(b, Tensor) else b_raw.dtype == torch.uint8
+        if not (precision_config.b_mx_scale is not None and b_packed):
+            # weights that are not MXFP4 (16-bit, or MXFP8, which is dequantised to bfloat16 below): the activations are
+            # dequantised, as the reference's own reference path does (matmul.py:772-778) -- exactly, to the type the
+            # product is computed in -- and take the kernel for 16-bit operands; no block scales are left
+            from .numerics_details.mxfp import upcast_from_mxfp
+            _lib.require_gpu(a_raw, "a")
+            a = upcast_from_mxfp(a_raw, a_mx_scale, torch.float16 if b_raw.dtype == torch.float16 else torch.bfloat16,
+                                 axis=-1)
+            a_mx_scale = None
+        elif a_fp4:
+            a = _widen_mxfp4_activations(a_raw)
     flex = precision_config.flex_ctx
     if flex.acc_data.scale is not None:
         raise NotImplementedError("accumulator flex scale is not built")
@@ -193,8 +223,8 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         w8 = b_data
         if w8.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2) or b_scale_cdna4:
             raise NotImplementedError("microscaled weights are built as MXFP4, or MXFP8 with scales in the strided layout")
-        if a.dtype != torch.bfloat16 or a_mx_scale is not None:
-            raise NotImplementedError("MXFP8 weights are built for bfloat16 activations")
+        if a.dtype != torch.bfloat16:
+            raise NotImplementedError("MXFP8 weights are built for bfloat16 or microscaled activations")
         from .numerics_details.mxfp import upcast_from_mxfp
         b_data = upcast_from_mxfp(w8, b_scale, torch.bfloat16, axis=-2)
         b_shape = list(b_data.shape)
@@ -237,7 +267,7 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         n_slices = batch = 1
     red_n = fused_activation.specs.reduction_n
     # microscaled activations stand for bf16 numbers (the reference dequantises them to bf16, matmul.py:772-778)
-    out_dtype = precision_config.out_dtype or (torch.bfloat16 if a_mx_scale is not None else a_dtype)
+    out_dtype = precision_config.out_dtype or (torch.bfloat16 if precision_config.a_mx_scale is not None else a_dtype)
     if mx_out:
         out_dtype = precision_config.out_dtype or (c.dtype if c is not None else torch.float8_e4m3fn)
         if out_dtype != torch.float8_e4m3fn:
