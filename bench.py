@@ -238,7 +238,9 @@ def run_dense(args, cfg, name):
     x, bias = x_cpu.to(dev), bias_cpu.to(dev)
     pc = PrecisionConfig(b_mx_scale=scales_for_matmul(scales, args.scale_layout), b_microblock_size=32)
     wq = weights_for_matmul(vals, args.value_layout)
-    y, kernel_ms, wall = timed(lambda: matmul(x, wq, bias, precision_config=pc), args.steps, args.warmup)
+    from triton_amd.matmul_details.opt_flags import scoped_opt_flags_constraints
+    with scoped_opt_flags_constraints({"block_m": args.block_m} if args.block_m else {}):
+        y, kernel_ms, wall = timed(lambda: matmul(x, wq, bias, precision_config=pc), args.steps, args.warmup)
     flops = 2.0 * M * K * N
     alg_bytes = M * K * 2 + K // 2 * N + K // 32 * N + N * 2 + M * N * 2
     torch.set_num_threads(os.cpu_count())

@@ -5,7 +5,10 @@
 
 namespace tamd {
 int dispatch_mm_f16(const tamd_matmul_args &a, int block_m, int grid_m, hipStream_t st) {
-  if (block_m == 0 && a.M <= 256 && stream16_applicable(a)) {
+  if (block_m == 0 && dense_prefers_k_groups(a)) {
+    block_m = 32;
+    grid_m = ((a.M + 31) / 32) * a.n_experts;
+  } else if (block_m == 0 && a.M <= 256 && stream16_applicable(a)) {
     // dense with few rows: row blocks of 16 through the streaming kernel (every CU busy, weights re-read from L2)
     block_m = 16;
     grid_m = ((a.M + 15) / 16) * a.n_experts;

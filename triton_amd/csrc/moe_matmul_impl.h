@@ -34,6 +34,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x8_t __attribute__((ext_vector_type(8)));
 
 constexpr bool is_fp8(int dt) { return dt == TAMD_FP8_E4M3 || dt == TAMD_FP8_E5M2; }
@@ -369,15 +370,45 @@ struct PipeShape {
   int scr_bytes;     // ring-mode scale ring: db stages x 4 waves x 1 KB
   int bytes;
 };
-constexpr PipeShape pipe_shape(bool fp8, bool ring, int lds_rows) {
+// "Deep mode" (16-bit path with the scales staged in LDS, row blocks of at most 64 rows): counted waits with three or
+// four activation stages and two weight stages.  With so few rows a stage's MFMAs take less time than a copy needs
+// to arrive, and the K loop of the two-stage pipeline runs at the latency of the copies.
+// K groups (KS = 2 or 4, row blocks of at most 32 rows): KS groups of four waves share a tile, each taking a
+// contiguous part of K through a pipeline of its own; their partial sums meet in LDS.  A problem with fewer tiles than
+// the part has CUs is bound by what one wave per SIMD can issue (a copy instruction holds its wave for about a
+// hundred cycles); more waves per SIMD fill those gaps.
+constexpr bool deep_mode(bool fp8, int lds_rows) { return !fp8 && lds_rows <= 64; }
+constexpr PipeShape pipe_shape(bool fp8, bool ring, int lds_rows, bool deep = false, int ks = 1) {
   PipeShape p{};
-  p.da = ring && lds_rows <= 64 ? 3 : 2;
-  p.db = ring ? 2 : 1;
+  p.da = deep ? (ks == 4 ? 3 : (lds_rows <= 32 ? 4 : 3)) : (ring && lds_rows <= 64 ? 3 : 2);
+  p.db = (ring || deep) && ks != 4 ? 2 : 1;
   p.as_bytes = fp8 ? p.da * 4 * (lds_rows < 64 ? 64 : lds_rows) * 4 : 0;
   p.scr_bytes = ring ? p.db * 4 * 1024 : 0;
   p.bytes = p.da * lds_rows * 128 + p.db * B_BYTES + p.as_bytes + p.scr_bytes;
   return p;
 }
+
+// Copies that a stage of the counted-wait loop (deep mode) may leave in flight.  The requests are made in this order:
+// stage j -- the stages before 0 are the loop's prologue -- asks for the activations of stage j + DA - 1 (NA copies)
+// and, if j is even, after them for the weights of pair j/2 + DB (NB copies).  A stage needs its own activations and,
+// if it is even, its pair's weights; copies complete in the order of their requests, so everything requested after
+// the last of those may still be outstanding when the stage begins.
+constexpr int ring_outstanding(int DA, int DB, int NA, int NB, bool odd) {
+  const int s = 64 + (odd ? 1 : 0);   // any stage in the steady state
+  int pos = 0, need_end = 0;
+  for (int j = 0; j < s; ++j) {
+    pos += NA;
+    if (j + DA - 1 == s) need_end = pos;
+    if (j % 2 == 0) {
+      pos += NB;
+      if (!odd && j / 2 + DB == s / 2 && pos > need_end) need_end = pos;
+    }
+  }
+  return pos - need_end;
+}
+static_assert(ring_outstanding(4, 2, 1, 4, false) == 6 && ring_outstanding(4, 2, 1, 4, true) == 10, "ring bookkeeping");
+static_assert(ring_outstanding(3, 2, 2, 4, false) == 6 && ring_outstanding(3, 2, 2, 4, true) == 6, "ring bookkeeping");
+static_assert(ring_outstanding(3, 1, 1, 4, false) == 1 && ring_outstanding(3, 1, 1, 4, true) == 5, "ring bookkeeping");
 
 // Epilogue of one output tile (shared by every tiled kernel).  The accumulators hold, for fragment
 // (i, f), element j: row 32i + 8(j/4) + 4h + j%4, column t.n0 + wave*64 + c32*NF + f.
@@ -703,8 +734,8 @@ TAMD_DEVICE late_args_t &kernel_args_late() {
 // a lane ends up with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3.
 // The wave reads them into registers at the start of the even stage and immediately requests the
 // next 128 K into the same region, so weights need no second buffer and no barrier.
-template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS>
-TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds) {
+template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS, int KS = 1>
+TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds_wg) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
   constexpr bool FP8 = is_fp8(XDT);
@@ -712,17 +743,31 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   constexpr int KA = A_ROW_BYTES / ESZ;       // K per activation stage
   constexpr int A_STAGE = LDS_ROWS * A_ROW_BYTES;
   constexpr bool RING = FP8 && !SC_LDS;
-  constexpr PipeShape PS = pipe_shape(FP8, RING, LDS_ROWS);
+  constexpr bool DEEP = SC_LDS && deep_mode(FP8, LDS_ROWS);
+  static_assert(KS == 1 || (DEEP && NFR == 1 && (KS == 2 || KS == 4)), "K groups: deep mode, one row fragment");
+  constexpr PipeShape PS = pipe_shape(FP8, RING, LDS_ROWS, DEEP, KS);
   constexpr int DA = PS.da, DB = PS.db;
   auto a_slot = [](int it) { return DA == 2 ? (it & 1) : it % DA; };
   constexpr uint32_t kOob = 0x7FFFFFFFu;
   const int tid = threadIdx.x;
-  const int wave = tid / kWave, lane = tid % kWave;
+  // K group of the wave (0 unless KS > 1) and its place among the group's four waves
+  const int grp = KS > 1 ? __builtin_amdgcn_readfirstlane(tid / 256) : 0;
+  const int wave = KS > 1 ? __builtin_amdgcn_readfirstlane((tid / kWave) & 3) : tid / kWave, lane = tid % kWave;
   const int c32 = lane % 32, h = lane / 32;
   const int K = a.K, N = a.N, G = K / 32;
   // a wave whose 64 columns lie beyond N (last column tile) copies its share of the activations and keeps the
   // barriers, but neither fetches weights nor runs MFMAs
   const bool wave_live = t.n0 + wave * 64 < N;
+  // the pipeline buffers of the wave's K group; the tile's scale image behind the last group's is shared
+  constexpr int PIPE_G = PS.bytes;
+  uint8_t *lds = lds_wg + grp * PIPE_G;
+  // the group's part of K: whole 128-K pairs [sup0, sup0 + n_sup), the same number for every group (a group whose
+  // part reaches past K copies zeros there: out-of-range offsets)
+  const int n_kb_all = (K + KB - 1) / KB;
+  const int n_sup = (n_kb_all + KS - 1) / KS;
+  const int sup0 = grp * n_sup;
+  const int k0 = sup0 * KB;
+  const int k_hi = KS > 1 ? (k0 + n_sup * KB < K ? k0 + n_sup * KB : K) : K;
 
   const v4i_t rx = make_rsrc((const uint8_t *)a.x + (int64_t)t.z * a.x_stride_z * ESZ, kOob);
   const v4i_t rw = make_rsrc((const uint8_t *)a.w + (int64_t)t.expert * a.w_stride_e, kOob);
@@ -734,7 +779,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   // per row; a copy always writes 64 dwords (lanes past the tile's rows write zeros)
   constexpr int AS_ROWS = LDS_ROWS < 64 ? 64 : LDS_ROWS;
   constexpr int AS_BYTES = PS.as_bytes;
-  uint8_t *lds_sc = lds + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
+  uint8_t *lds_sc = KS > 1 ? lds_wg + KS * PIPE_G : lds + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
 
   // ---- scales of the whole tile, once.  Strided: 256 columns x G bytes, contiguous in memory.  CDNA4
   // pre-shuffle: the tile's 8 blocks of 32 columns are contiguous too (KSP*32 bytes each); byte
@@ -751,14 +796,15 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       // by DMA, 1 KB per instruction: in flight together with the first activation / weight stages and
       // awaited with them at the first barrier of the K loop
       const v4i_t rs = make_rsrc(sc_src, (uint32_t)sc_avail);
-      const uint32_t lds_sc_addr = lds_base + DA * A_STAGE + DB * B_BYTES + AS_BYTES;
-      for (int i = wave; i * 1024 < sc_tile_bytes; i += 4) dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
+      const uint32_t lds_sc_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds_sc;
+      for (int i = wave + 4 * grp; i * 1024 < sc_tile_bytes; i += 4 * KS)
+        dma16(rs, lds_sc_addr + i * 1024, i * 1024 + lane * 16, 0);
     } else {
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)sc_src, 0, (uint32_t)(tile_cols * G),
                                                                         0x00020000);
       const int n_dw = (BLOCK_N * G + 3) / 4;
       const int avail = tile_cols * G;
-      for (int i = tid; i < n_dw; i += 256) {
+      for (int i = tid; i < n_dw; i += 256 * KS) {
         uint32_t v;
         if (i * 4 + 4 <= avail || i * 4 >= avail) {
           v = __builtin_amdgcn_raw_buffer_load_b32(rs, i * 4, 0, 0);  // whole, or wholly outside (zeros)
@@ -863,25 +909,25 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   const int n_ka = (K + KA - 1) / KA;      // activation stages
   const int n_kb = (K + KB - 1) / KB;      // weight super-stages (two activation stages each)
   auto issue_a = [&](int it) {             // clamped: past the end the last stage is copied again
-    if constexpr (!RING) it = it < n_ka ? it : n_ka - 1;   // (ring mode: chunks past K are not read at all)
-    const int kb = it * KA;
-    const uint32_t akill = kb + a_chunk * (16 / ESZ) < K ? 0u : kOob;
+    if constexpr (!RING && !DEEP) it = it < n_ka ? it : n_ka - 1;   // (ring / deep mode: chunks past K are not read at all)
+    const int kb = k0 + it * KA;
+    const uint32_t akill = kb + a_chunk * (16 / ESZ) < k_hi ? 0u : kOob;
     const uint32_t sb = lds_base + a_slot(it) * A_STAGE + wave * 8 * A_ROW_BYTES;
 #pragma unroll
     for (int i = 0; i < NFR; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * ESZ);
   };
   auto issue_b = [&](int sup) {
     const uint32_t region = DB == 2 ? (uint32_t)(sup & 1) * B_BYTES : 0u;
-    if constexpr (!RING) sup = sup < n_kb ? sup : n_kb - 1;
-    const int kb = sup * KB;
+    if constexpr (!RING && !DEEP) sup = sup < n_kb ? sup : n_kb - 1;
+    const int kb = k0 + sup * KB;
     if (wnat) {   // one 4 KB block, copied as it lies
-      dma16_x4(rw, lds_b + region, w_off[0] | ((wave_live && kb < K) ? 0u : kOob), (uint32_t)sup << 12);
+      dma16_x4(rw, lds_b + region, w_off[0] | ((wave_live && kb < k_hi) ? 0u : kOob), (uint32_t)(sup0 + sup) << 12);
       return;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t bkill = (wave_live && kb + w_kpart(j) < K) ? 0u : kOob;
-      dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, (uint32_t)sup << w_stage_shift);
+      const uint32_t bkill = (wave_live && kb + w_kpart(j) < k_hi) ? 0u : kOob;
+      dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, (uint32_t)(sup0 + sup) << w_stage_shift);
     }
   };
   // Paired form (ring mode, row blocks of up to 64 rows): the weights of stages 2p and 2p + 1 are 128 contiguous bytes
@@ -977,7 +1023,9 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         // (groups past the end of K meet zero codes and zero activations; their scale only has to be some finite
         // value of this column).  Pre-shuffled: byte 256*(kg/8) + 64*(kg%4) + 2*((kg%8)/4); the padding up to a
         // multiple of 8 groups is stored (zeros), so nothing is clamped.
-        const int sup_off = cdna4 ? (sup >> 1) * 256 + (sup & 1) * 2 : sup * 4;  // wave uniform
+        // (K groups: a group's pairs past the end of K hold zero codes and meet the last pair's scales)
+        const int sg = KS > 1 ? (sup0 + sup < n_kb_all ? sup0 + sup : n_kb_all - 1) : sup;
+        const int sup_off = cdna4 ? (sg >> 1) * 256 + (sg & 1) * 2 : sg * 4;  // wave uniform
         int kg_off = sup_off + sc_lane_off[q];
         kg_off = kg_off < sc_clamp ? kg_off : sc_clamp;
         uint32_t sbyte;
@@ -1154,6 +1202,34 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       issue_b(it + 1);
       compute(it, Set0{}, Set0{});
     }
+  } else if constexpr (DEEP) {
+    // Stage s requests the activations of stage s + DA - 1, an even stage after them the weights of pair s/2 + DB
+    // (a weight region is free once its pair's weights are in registers).  Copies complete in the order of their
+    // requests: a stage waits until only the requests made after the ones it needs are outstanding
+    // (ring_outstanding).  The requests before the loop are those of the stages before 0, in the same order, so the
+    // counts hold from the first stage on.
+    constexpr int PRE = DA - 1 > 2 * DB ? DA - 1 : 2 * DB;
+#pragma unroll
+    for (int j = -PRE; j < 0; ++j) {
+      if (j + DA - 1 >= 0) issue_a(j + DA - 1);
+      if (j % 2 == 0 && j / 2 + DB >= 0) issue_b(j / 2 + DB);
+    }
+    const int n_stage = KS > 1 ? 2 * n_sup : n_ka;   // (K groups: the same trip count, and barriers, for every group)
+    for (int it = 0; it < n_stage; it += 2) {
+      wait_vmcnt<ring_outstanding(DA, DB, NFR, 4, false)>();
+      __syncthreads();
+      load_b(it >> 1, Set0{});
+      issue_a(it + DA - 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // weights are in registers: the region may be refilled
+      issue_b((it >> 1) + DB);
+      compute(it, Set0{}, Set0{});
+      if (it + 1 < n_stage) {
+        wait_vmcnt<ring_outstanding(DA, DB, NFR, 4, true)>();
+        __syncthreads();
+        issue_a(it + DA);
+        compute(it + 1, Set1{}, Set0{});
+      }
+    }
   } else {
     for (int it = 0; it < n_ka; it += 2) {
       wait_dma();
@@ -1176,7 +1252,37 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   wait_dma();
 
-  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT, FP8>(kernel_args_late(), t, acc, lds);
+  if constexpr (KS > 1) {
+    // The groups' partial sums meet in LDS (the pipelines are dead: after the barrier every copy has landed and every
+    // operand has been read): group g > 0 leaves its accumulators in plane g - 1 and ends; group 0 adds the planes in
+    // the order of the groups and finishes the tile alone (a barrier waits only for the waves that are still alive).
+    // (16 bytes per lane and access: a plane is [4 waves][NF x 4 quads][64 lanes] of four accumulators)
+    f32x4_t *red = (f32x4_t *)lds_wg;
+    constexpr int PLANE = 4 * NF * 4 * kWave;
+    __syncthreads();
+    if (grp > 0) {
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          red[(grp - 1) * PLANE + ((wave * NF + f) * 4 + j) * kWave + lane] =
+              f32x4_t{acc[0][f][4 * j], acc[0][f][4 * j + 1], acc[0][f][4 * j + 2], acc[0][f][4 * j + 3]};
+    }
+    __syncthreads();
+    if (grp > 0) return;
+#pragma unroll
+    for (int g = 1; g < KS; ++g)
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x4_t v = red[(g - 1) * PLANE + ((wave * NF + f) * 4 + j) * kWave + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[0][f][4 * j + e] += v[e];
+        }
+    __syncthreads();   // the epilogue stages its output through the same memory
+  }
+  tile_epilogue<NFR, ACT, FP8 ? TAMD_BF16 : XDT, FP8>(kernel_args_late(), t, acc, lds_wg);
 }
 
 // Row fragments a workgroup can hold: a 128-row block of 16-bit activations also takes a remainder of
@@ -1189,17 +1295,17 @@ struct TileShape {
 };
 
 // BM: block size of the ragged schedule the kernel consumes (16..128).
-template <int XDT, int BM, int ACT, bool SC_LDS>
+template <int XDT, int BM, int ACT, bool SC_LDS, int KS = 1>
 TAMD_DEVICE void tile_entry(const tamd_matmul_args &a, int grid_n, int64_t grid_total, int group_m, uint8_t *lds) {
   typedef TileShape<XDT, BM> S;
   Tile t;
-  if (group_m == 0) {  // the workgroup finds its tile's place itself (grid_total = row blocks of the launch)
+  if (KS == 1 && group_m == 0) {  // the workgroup finds its tile's place itself (grid_total = row blocks of the launch)
     if (!locate_tile_sorted<BM, S::EXTRA>(a, grid_n, (int)grid_total, t, lds)) return;
   } else if (!locate_tile<BM, S::EXTRA>(a, grid_n, grid_total, group_m, t)) return;
   const int nfr = (t.rows + 31) / 32;  // active row fragments (workgroup uniform)
-#define TAMD_CASE(n)                                                                 \
-  case n:                                                                            \
-    if constexpr (n <= S::MF) run_tile<XDT, n, S::LDS_ROWS, ACT, SC_LDS>(a, t, lds); \
+#define TAMD_CASE(n)                                                                     \
+  case n:                                                                                \
+    if constexpr (n <= S::MF) run_tile<XDT, n, S::LDS_ROWS, ACT, SC_LDS, KS>(a, t, lds); \
     break;
   switch (nfr) { TAMD_CASE(1) TAMD_CASE(2) TAMD_CASE(3) TAMD_CASE(4) TAMD_CASE(5) }
 #undef TAMD_CASE
@@ -1212,6 +1318,14 @@ __global__ __launch_bounds__(256, 2) void mm_x16_mxfp4_kernel(tamd_matmul_args a
   tile_entry<XDT, BM, ACT, SC_LDS>(a, grid_n, grid_total, group_m, lds);
 }
 
+// K groups: KS x 4 waves per tile of at most 32 rows, scales of the tile in LDS (see pipe_shape).
+template <int XDT, int BM, int ACT, int KS>
+__global__ __launch_bounds__(256 * KS, 1) void mm_x16_mxfp4_kgroups_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total,
+                                                                            int group_m) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  tile_entry<XDT, BM, ACT, true, KS>(a, grid_n, grid_total, group_m, lds);
+}
+
 template <int XDT, int BM, int ACT, bool SC_LDS>
 __global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a, int grid_n, int64_t grid_total,
                                                                  int group_m) {
@@ -1222,7 +1336,8 @@ __global__ __launch_bounds__(256, 2) void mm_x8_mxfp4_kernel(tamd_matmul_args a,
 template <int XDT, int BM, int ACT>
 int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   constexpr int LDS_ROWS = TileShape<XDT, BM>::LDS_ROWS;
-  constexpr int PIPE_BYTES = pipe_shape(is_fp8(XDT), false, LDS_ROWS).bytes;
+  constexpr bool DEEP = deep_mode(is_fp8(XDT), LDS_ROWS);   // (kernels with the scales in LDS)
+  constexpr int PIPE_BYTES = pipe_shape(is_fp8(XDT), false, LDS_ROWS, DEEP).bytes;
   constexpr int RING_BYTES = pipe_shape(is_fp8(XDT), true, LDS_ROWS).bytes;
   constexpr int OUT_BYTES = LDS_ROWS * (ACT == TAMD_ACT_SWIGLU ? 128 : 256) * 2;  // epilogue staging
   int grid_n = (a.N + BLOCK_N - 1) / BLOCK_N;
@@ -1238,15 +1353,16 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int64_t sc_bytes = (BLOCK_N * (cdna4 ? (G + 7) / 8 * 8 : G) + 1023) / 1024 * 1024;  // whole 1 KB copies
   const bool dense_sc = cdna4 || (a.w_mx_stride_k == 1 && a.w_mx_stride_n == G && a.w_mx_stride_e % 4 == 0 &&
                                   aligned(a.w_mx_scale, 4) && (BLOCK_N * G) % 4 == 0);
-  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= 80 * 1024 && !(is_fp8(XDT) && cdna4);
-  size_t lds_bytes = is_fp8(XDT) && !sc_in_lds ? RING_BYTES : PIPE_BYTES + (sc_in_lds ? sc_bytes : 0);
+  // (deep mode is worth a CU to itself: up to 156 KB; otherwise two workgroups have to fit)
+  const int sc_in_lds = dense_sc && PIPE_BYTES + sc_bytes <= (DEEP ? 156 : 80) * 1024 && !(is_fp8(XDT) && cdna4);
+  constexpr int PLAIN_BYTES = pipe_shape(is_fp8(XDT), false, LDS_ROWS).bytes;   // 16-bit path, scales read from memory
+  size_t lds_bytes = sc_in_lds ? PIPE_BYTES + sc_bytes : (is_fp8(XDT) ? RING_BYTES : PLAIN_BYTES);
   if (lds_bytes < (size_t)OUT_BYTES) lds_bytes = OUT_BYTES;
   void (*kern)(tamd_matmul_args, int, int64_t, int);
   if constexpr (is_fp8(XDT))
     kern = sc_in_lds ? mm_x8_mxfp4_kernel<XDT, BM, ACT, true> : mm_x8_mxfp4_kernel<XDT, BM, ACT, false>;
   else
     kern = sc_in_lds ? mm_x16_mxfp4_kernel<XDT, BM, ACT, true> : mm_x16_mxfp4_kernel<XDT, BM, ACT, false>;
-  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
   // row blocks walked together: as many as one expert (or batch entry) has, while their activation
   // rows (BM x K each) fit comfortably in one XCD's 4 MB L2
   const int64_t rows_per_slice = a.block_schedule ? a.M / a.n_experts : a.M;
@@ -1254,6 +1370,24 @@ int launch_x16_act(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   const int64_t fit = (int64_t)(2.5 * 1024 * 1024) / ((int64_t)BM * a.K * (is_fp8(XDT) ? 1 : 2));
   group_m = group_m > fit ? fit : group_m;
   group_m = group_m < 1 ? 1 : (group_m > 16 ? 16 : group_m);
+  if constexpr (!is_fp8(XDT) && BM == 32) {
+    // Fewer tiles than CUs: K groups, so that every SIMD of the CUs that do get a tile holds two to four waves
+    // (at least two 128-K pairs per group; the groups' pipelines and the tile's scales have to fit one CU's LDS)
+    int cus = 0;
+    if (int rc = cu_count(cus)) return rc;
+    const int64_t pairs = (a.K + KB - 1) / KB;
+    const int ks = total * 2 <= cus && pairs >= 8 ? 4 : (total <= cus && pairs >= 4 ? 2 : 1);
+    const size_t pipe = ks == 4 ? 4 * (size_t)pipe_shape(false, false, LDS_ROWS, true, 4).bytes
+                                : 2 * (size_t)pipe_shape(false, false, LDS_ROWS, true, 2).bytes;
+    if (ks > 1 && dense_sc && pipe + sc_bytes <= 156 * 1024) {
+      void (*kk)(tamd_matmul_args, int, int64_t, int) =
+          ks == 4 ? mm_x16_mxfp4_kgroups_kernel<XDT, BM, ACT, 4> : mm_x16_mxfp4_kgroups_kernel<XDT, BM, ACT, 2>;
+      if (int rc = raise_lds_limit_once((const void *)kk)) return rc;
+      kk<<<dim3((unsigned)launch), 256 * ks, pipe + sc_bytes, st>>>(a, grid_n, total, (int)group_m);
+      return launch_status();
+    }
+  }
+  if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
   if (a.block_schedule && a.block_offs && group_m == 1 && grid_m <= 1024) {
     // few row blocks per expert: the workgroups take the row blocks largest first, dealt evenly to the XCDs
     const int64_t sorted_launch = (int64_t)((grid_m + 7) / 8) * 8 * grid_n;
@@ -1273,6 +1407,16 @@ inline int dense_block_m(const tamd_matmul_args &a) {
   for (int bm : cand)
     if (a.M > bm / 2 && (a.M + bm - 1) / bm * cols >= 256) return bm;
   return 16;  // too few tiles either way: the smallest block gives the most
+}
+// A dense / batched problem of 161 to 256 rows whose 32-row tiles number at most half the CUs and whose K holds at
+// least eight 128-K pairs: faster as 32-row tiles with four K groups each (256 x 2048 x 4096: 14.6 us) than as 16-row
+// blocks through the streaming kernel (22 us), which is what problems of fewer rows take.
+inline bool dense_prefers_k_groups(const tamd_matmul_args &a) {
+  if (is_fp8(a.x_dtype) || a.M <= 160 || a.M > 256 || (a.K + KB - 1) / KB < 8) return false;
+  int cus = 0;
+  if (cu_count(cus) != 0) return false;
+  const int64_t tiles = (int64_t)((a.M + 31) / 32) * a.n_experts * ((a.N + BLOCK_N - 1) / BLOCK_N);
+  return tiles * 2 <= cus;
 }
 inline void dense_grid(const tamd_matmul_args &a, int &block_m, int &grid_m) {
   if (block_m != 0) return;

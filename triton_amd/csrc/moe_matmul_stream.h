@@ -26,8 +26,6 @@
 
 namespace tamd {
 
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
 template <int XDT>
 struct Mma16;
 template <>
