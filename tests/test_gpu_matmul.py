@@ -237,12 +237,15 @@ def test_fp8_ragged(block_m, do_gather, do_scatter, do_gamma, act, fp8, device):
 
 @pytest.mark.parametrize("block_m", [32, 64, 128])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float8_e4m3fn])
-def test_fp8_ragged_long_k_strided_scales(block_m, out_dtype, device):
+@pytest.mark.parametrize("K", [4608, 6432])
+def test_fp8_ragged_long_k_strided_scales(block_m, out_dtype, K, device):
     """K = 4608 with strided scales: a tile's scales (256 columns x 144 bytes) no longer fit LDS beside the pipeline of a
-    128-row block, so they travel with the weight stages (byte-sized copies); smaller blocks still stage them.  Also the
-    plain float8_e4m3fn output of fp8-row kernels (the rows the next matmul of a layer consumes)."""
+    128-row block, so they travel with the weight stages (byte-sized copies); smaller blocks still stage them.
+    K = 6432 (201 groups): no block size can stage them, so row blocks of up to 64 rows run the paired ring loop with
+    strided scales, over an odd number of stages (51) whose last holds a single group.  Also the plain
+    float8_e4m3fn output of fp8-row kernels (the rows the next matmul of a layer consumes)."""
     torch.manual_seed(3)
-    E, K, N, M = 3, 4608, 264, 300
+    E, N, M = 3, 264, 300
     sizes = torch.tensor([130, 0, 170], dtype=torch.int32)
     x8, xs = to_fp8(torch.randn(M, K), torch.float8_e4m3fn)
     w = torch.randn(E, K, N) * 0.02
@@ -684,6 +687,38 @@ def test_mxfp8_activations_ragged(block_m, cdna4_scales, device):
                      precision_config=pc, gammas=gammas.to(device), fused_activation=swiglu_act(1.702, 7.0), c=out_init)
     ref = MR.matmul_ref(rq, rv, bias, slice_sizes=sizes, gather_indx=gather, scatter_indx=scatter, a_mx_scale=rxs,
                         b_mx_scale=rs, gammas=gammas, fused_swiglu=(1.702, 7.0))
+    check(out, ref)
+
+
+# ---------------------------------------------------------------------------- K groups (few 32-row tiles)
+
+
+@pytest.mark.parametrize("K", [512, 1440, 2880])        # 4, 11.25 and 22.5 pairs of 128: two and four K groups, ragged ends
+@pytest.mark.parametrize("mode", ["dense", "ragged", "batched"])
+@pytest.mark.parametrize("cdna4", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_k_groups(K, mode, cdna4, dtype, device):
+    """Row blocks of 32 with fewer tiles than CUs: the tile's K range is shared by groups of four waves whose partial
+    sums meet in LDS.  The last group's part ends inside a pair (K = 1440, 2880) or holds no K at all."""
+    torch.manual_seed(K)
+    N = 400 if not cdna4 else 448
+    E = 3
+    act = mode != "batched"
+    if mode == "dense":
+        x, w, bias, sizes = torch.randn(70, K), torch.randn(K, N) * 0.05, torch.randn(N), None
+    elif mode == "ragged":
+        sizes = torch.tensor([33, 0, 30], dtype=torch.int32)
+        x, w, bias = torch.randn(63, K), torch.randn(E, K, N) * 0.05, torch.randn(E, N)
+    else:
+        x, w, bias, sizes = torch.randn(E, 40, K), torch.randn(E, K, N) * 0.05, torch.randn(E, N), None
+    x = x.to(dtype)
+    v, s, rv, rs = quantize_w(w, device)
+    pc = PrecisionConfig(b_mx_scale=preshuffle(s) if cdna4 else s, b_microblock_size=32)
+    md = make_ragged_tensor_metadata(sizes.to(device), 63) if mode == "ragged" else None
+    with scoped_opt_flags_constraints({"block_m": 32}):
+        out = matmul(x.to(device), in_blocks(v) if cdna4 else v, bias.to(device), md, precision_config=pc,
+                     fused_activation=swiglu_act(1.702, 7.0) if act else None)
+    ref = MR.matmul_ref(x, rv, bias, slice_sizes=sizes, b_mx_scale=rs, fused_swiglu=(1.702, 7.0) if act else None)
     check(out, ref)
 
 

@@ -853,10 +853,17 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       as_off = src * (uint32_t)a.x_mx_stride_m;
     }
   }
+  // Copies per request, as the counted waits of the ring loops below see them (a wave's copies complete in the order
+  // of their requests): the loops of the issue_* functions run to these numbers and the waits are written in them.
+  constexpr int CP_A = NFR;        // issue_a: one copy per row fragment
+  constexpr int CP_AS = 4;         // issue_as: one per 32-K group of the stage (waves that hold rows only)
+  constexpr int CP_B = 4;          // issue_b: four 1 KB pieces
+  constexpr int CP_BPAIR = 8;      // issue_b_pair: eight
+  constexpr int CP_SC_STRIDED = 4; // issue_sc: one per group with strided scales, one in all when pre-shuffled
   auto issue_as = [&](int it) {
     if (x_mx && wave * 64 < LDS_ROWS) {
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4)
+      for (int g4 = 0; g4 < CP_AS; ++g4)
         dma1(ras, lds_as + (a_slot(it) * 4 + g4) * AS_ROWS * 4 + wave * 256, it * 4 + g4 < G ? as_off : kOob,
              (uint32_t)(it * 4 + g4));
     }
@@ -914,18 +921,19 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     const uint32_t akill = kb + a_chunk * (16 / ESZ) < k_hi ? 0u : kOob;
     const uint32_t sb = lds_base + a_slot(it) * A_STAGE + wave * 8 * A_ROW_BYTES;
 #pragma unroll
-    for (int i = 0; i < NFR; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * ESZ);
+    for (int i = 0; i < CP_A; ++i) dma16(rx, sb + i * 32 * A_ROW_BYTES, a_off[i] | akill, kb * ESZ);
   };
   auto issue_b = [&](int sup) {
     const uint32_t region = DB == 2 ? (uint32_t)(sup & 1) * B_BYTES : 0u;
     if constexpr (!RING && !DEEP) sup = sup < n_kb ? sup : n_kb - 1;
     const int kb = k0 + sup * KB;
+    static_assert(CP_B == 4, "dma16_x4 makes four copies");
     if (wnat) {   // one 4 KB block, copied as it lies
       dma16_x4(rw, lds_b + region, w_off[0] | ((wave_live && kb < k_hi) ? 0u : kOob), (uint32_t)(sup0 + sup) << 12);
       return;
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < CP_B; ++j) {
       const uint32_t bkill = (wave_live && kb + w_kpart(j) < k_hi) ? 0u : kOob;
       dma16(rw, lds_b + region + j * 1024, w_off[j] | bkill, (uint32_t)(sup0 + sup) << w_stage_shift);
     }
@@ -953,6 +961,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   auto issue_b_pair = [&](int pair) {
     if constexpr (PAIRED) {
       const int kb = pair * 256;
+      static_assert(CP_BPAIR == 8, "two dma16_x4, or eight copies of 128 bytes per column");
       if (wnat) {
         // block layout: the pair's two stages are two 4 KB blocks, copied as they lie (first stage, then second)
         dma16_x4(rw, lds_b2, w_off[0] | ((wave_live && kb < K) ? 0u : kOob), (uint32_t)(2 * pair) * 4096u);
@@ -960,7 +969,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         return;
       }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < CP_BPAIR; ++j) {
         const uint32_t bkill = (wave_live && kb + w2_part[j] * 32 < K) ? 0u : kOob;
         dma16(rw, lds_b2 + j * 1024, w2_off[j] | bkill, kb >> 1);
       }
@@ -992,7 +1001,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         dma16(rsc, dst, sup * 4 < G ? scr_voff : kOob, (uint32_t)(256 * (sup >> 1)));
       } else {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
+        for (int g4 = 0; g4 < CP_SC_STRIDED; ++g4) {
           const int kg = sup * 4 + g4;
           dma1(rsc, dst + g4 * 256, kg < G ? scr_voff : kOob, (uint32_t)((int64_t)kg * a.w_mx_stride_k));
         }
@@ -1136,7 +1145,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     // Copies complete in the order of their requests, so a stage waits by count for what it needs and leaves the
     // later requests in flight.
     const bool as_wave = x_mx && wave * 64 < LDS_ROWS;
-    constexpr int NSC = 4;  // scale copies of a stage with strided scales (1 when pre-shuffled)
+    constexpr int NSC = CP_SC_STRIDED;  // scale copies of a stage with strided scales (1 when pre-shuffled)
     if constexpr (PAIRED) {
       // Three activation stages; an even stage s moves the weights of s and s + 1 into registers and requests those of
       // s + 2 and s + 3 (one pair), the odd stage requests only activations.
@@ -1145,7 +1154,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       issue_a(1), issue_as(1);
       for (int it = 0; it < n_ka; it += 2) {
         // in flight at most: the activations of stage it + 1
-        if (as_wave) wait_vmcnt<NFR + 4>(); else wait_vmcnt<NFR>();
+        if (as_wave) wait_vmcnt<CP_A + CP_AS>(); else wait_vmcnt<CP_A>();
         __syncthreads();
         load_b(it, Set0{});
         load_b(it + 1, Set1{});
@@ -1158,8 +1167,8 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
         compute(it, Set0{}, Set0{});
         if (it + 1 < n_ka) {
           // in flight at most: everything the even stage requested
-          if (cdna4) { if (as_wave) wait_vmcnt<NFR + 4 + 8 + 2>(); else wait_vmcnt<NFR + 8 + 2>(); }
-          else { if (as_wave) wait_vmcnt<NFR + 4 + 8 + 2 * NSC>(); else wait_vmcnt<NFR + 8 + 2 * NSC>(); }
+          if (cdna4) { if (as_wave) wait_vmcnt<CP_A + CP_AS + CP_BPAIR + 2>(); else wait_vmcnt<CP_A + CP_BPAIR + 2>(); }
+          else { if (as_wave) wait_vmcnt<CP_A + CP_AS + CP_BPAIR + 2 * NSC>(); else wait_vmcnt<CP_A + CP_BPAIR + 2 * NSC>(); }
           __syncthreads();
           fp8_read0(it + 1);
           issue_a(it + 3);
@@ -1174,7 +1183,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       issue_b(0), issue_sc(0);
       issue_a(0), issue_as(0), issue_b(1), issue_sc(1);
       for (int it = 0; it < n_ka; ++it) {
-        if (cdna4) wait_vmcnt<4 + 1>(); else wait_vmcnt<4 + NSC>();
+        if (cdna4) wait_vmcnt<CP_B + 1>(); else wait_vmcnt<CP_B + NSC>();
         __syncthreads();
         load_b(it, Set0{});
         fp8_read0(it);
@@ -1216,7 +1225,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
     }
     const int n_stage = KS > 1 ? 2 * n_sup : n_ka;   // (K groups: the same trip count, and barriers, for every group)
     for (int it = 0; it < n_stage; it += 2) {
-      wait_vmcnt<ring_outstanding(DA, DB, NFR, 4, false)>();
+      wait_vmcnt<ring_outstanding(DA, DB, CP_A, CP_B, false)>();
       __syncthreads();
       load_b(it >> 1, Set0{});
       issue_a(it + DA - 1);
@@ -1224,7 +1233,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       issue_b((it >> 1) + DB);
       compute(it, Set0{}, Set0{});
       if (it + 1 < n_stage) {
-        wait_vmcnt<ring_outstanding(DA, DB, NFR, 4, true)>();
+        wait_vmcnt<ring_outstanding(DA, DB, CP_A, CP_B, true)>();
         __syncthreads();
         issue_a(it + DA);
         compute(it + 1, Set1{}, Set0{});
@@ -1242,7 +1251,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       if (it + 1 < n_ka) {
         // the weight copies just issued (4, after the activation stage it + 1) are not needed before the next
         // even stage and take the longest (weights stream from HBM, activations mostly hit L2): leave them in flight
-        wait_vmcnt<4>();
+        wait_vmcnt<CP_B>();
         __syncthreads();
         issue_a(it + 2);
         compute(it + 1, Set1{}, Set0{});
