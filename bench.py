@@ -255,7 +255,10 @@ def run_dense(args, cfg, name):
                     value_layout=args.value_layout)
     out["matmul_kernel_tflops"] = round(flops / (kernel_ms * 1e-3) / 1e12, 2)
     out["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "mm_stream16_kernel",
+                       "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                       # 161-256 rows: 32-row tiles shared by four K groups; fewer rows or a forced block of 16: streaming kernel
+                       "kernel": "mm_x16_mxfp4_kgroups_kernel" if 160 < M <= 256 and args.block_m in (0, None, 32)
+                       else ("mm_stream16_kernel" if args.block_m in (0, None, 16) else "mm_x16_mxfp4_kernel"),
                        "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": alg_bytes, "algorithmic_flops": flops,
                        "note": "event pairs around one call include its host time; the problem is latency bound "
                                "(4.3 GFLOP, 7.6 MB)"}

@@ -690,6 +690,33 @@ def test_mxfp8_activations_ragged(block_m, cdna4_scales, device):
     check(out, ref)
 
 
+# ---------------------------------------------------------------------------- weights in the kernels' block layout
+
+
+@pytest.mark.parametrize("kind", ["tiled_bf16", "stream_bf16", "tiled_fp8", "k_groups"])
+def test_block_layout_gives_the_same_bits(kind, device):
+    """The 4 KB blocks hold a wave's LDS image as it is: the kernels do the same arithmetic in the same order from either
+    layout, so the outputs are bit for bit the same (K and N ragged against the blocks: 2880 = 22.5 x 128, 400 = 6.25 x 64)."""
+    torch.manual_seed(5)
+    E, K, N = 4, 2880, 400
+    rows = {"tiled_bf16": [150, 0, 33, 7], "stream_bf16": [3, 0, 9, 1], "tiled_fp8": [150, 0, 33, 7], "k_groups": [30, 20, 0, 5]}[kind]
+    sizes = torch.tensor(rows, dtype=torch.int32)
+    M = int(sizes.sum())
+    w = torch.randn(E, K, N) * 0.03
+    bias = torch.randn(E, N)
+    v, s, rv, rs = quantize_w(w, device)
+    md = make_ragged_tensor_metadata(sizes.to(device), M)
+    if kind == "tiled_fp8":
+        x8, xs = to_fp8(torch.randn(M, K), torch.float8_e4m3fn)
+        x, pc = x8.to(device), fp8_pc(s, xs, device, torch.bfloat16, torch.float8_e4m3fn)
+    else:
+        x, pc = torch.randn(M, K).to(torch.bfloat16).to(device), PrecisionConfig(b_mx_scale=s, b_microblock_size=32)
+    with scoped_opt_flags_constraints({"block_m": 32} if kind == "k_groups" else {}):
+        y_strided = matmul(x, v, bias.to(device), md, precision_config=pc, fused_activation=swiglu_act(1.702, 7.0))
+        y_blocks = matmul(x, in_blocks(v), bias.to(device), md, precision_config=pc, fused_activation=swiglu_act(1.702, 7.0))
+    assert torch.equal(y_strided.view(torch.int16), y_blocks.view(torch.int16))
+
+
 # ---------------------------------------------------------------------------- K groups (few 32-row tiles)
 
 
