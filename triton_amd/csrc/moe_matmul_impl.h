@@ -724,16 +724,20 @@ TAMD_DEVICE late_args_t &kernel_args_late() {
 }
 
 // One output tile with NFR (compile time) active 32-row fragments.
-// LDS: [A stage 0 | A stage 1 | B: 4 wave-private regions | (fp8) activation block scales, 2 stages | e8m0 scales of the tile].
+// LDS: [A stages (2 to 4) | B: 4 wave-private regions, one or two stages | (fp8) activation block scales | scale ring or
+// the e8m0 scales of the whole tile]; with K groups (KS > 1) one such pipeline per group, the tile's scales behind them.
 //
-// Both operands reach LDS by DMA.  Activations: 64 K per stage, double buffered; wave w copies rows
+// Both operands reach LDS by DMA.  Activations: 64 K per stage (128 K of fp8); wave w copies rows
 // 8w..8w+7 of every 32-row fragment (8 lanes x 16 B per row); chunk c of row r sits at slot
 // c ^ ((r>>1)&7), which makes the 32-row MFMA operand reads bank-conflict free.  Weights: every
-// second stage each wave copies 64 contiguous bytes (128 K) of each of its own 64 columns into
-// its private region, position p' = f*32 + c holding global column 2c + f of the wave's strip (so
-// a lane ends up with a gate/linear column pair), the four 16-byte parts rotated by (p'>>2)&3.
-// The wave reads them into registers at the start of the even stage and immediately requests the
-// next 128 K into the same region, so weights need no second buffer and no barrier.
+// second stage (every stage of fp8) each wave copies 128 K of its own 64 columns into its private region: position
+// p' = f*32 + c holds global column 2c + f of the wave's strip (so a lane ends up with a gate/linear column pair), the
+// four 16-byte parts rotated by ((p'>>2)&3) ^ 2f.  From column-strided weights that is 64 contiguous bytes of each
+// column; weights in the block layout (TAMD_W_CDNA4_BLOCKS) hold exactly this image, 4 KB per strip and 128 K, and
+// are copied as they lie.  The wave reads the region into registers at the start of the stage and immediately
+// requests the next 128 K into it, so weights need no barrier.
+// Loops: two stages and full waits (16-bit, row blocks above 64 rows or scales not in LDS); counted waits over a
+// deeper ring (deep mode, K groups: 16-bit; ring mode, paired: fp8), see pipe_shape.
 template <int XDT, int NFR, int LDS_ROWS, int ACT, bool SC_LDS, int KS = 1>
 TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds_wg) {
   typedef Mma<XDT> M;
@@ -1141,6 +1145,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
 
   typedef std::integral_constant<int, 0> Set0;
   typedef std::integral_constant<int, 1> Set1;
+  uint32_t warm = 0;   // (K groups: a byte fetched only to warm the caches, see below)
   if constexpr (RING) {
     // Copies complete in the order of their requests, so a stage waits by count for what it needs and leaves the
     // later requests in flight.
@@ -1212,6 +1217,16 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
       compute(it, Set0{}, Set0{});
     }
   } else if constexpr (DEEP) {
+    if constexpr (KS > 1) {
+      // A K-group tile's fixed costs are a third of its time, so the first thing its epilogue fetches -- the bias of the
+      // lane's columns -- is requested here already.  The request is older than every copy (the counted waits cover
+      // it) and only warms the caches: the byte is dropped after the loop.
+      if (a.bias && grp == 0) {
+        const int esz = a.bias_dtype == TAMD_F32 ? 4 : 2;
+        const uint8_t *bp = (const uint8_t *)a.bias + (col0 < N ? ((int64_t)t.expert * a.bias_stride_e + col0) * esz : 0);
+        asm volatile("global_load_ubyte %0, %1, off" : "=v"(warm) : "v"(bp) : "memory");
+      }
+    }
     // Stage s requests the activations of stage s + DA - 1, an even stage after them the weights of pair s/2 + DB
     // (a weight region is free once its pair's weights are in registers).  Copies complete in the order of their
     // requests: a stage waits until only the requests made after the ones it needs are outstanding
@@ -1260,6 +1275,7 @@ TAMD_DEVICE void run_tile(const tamd_matmul_args &a, const Tile &t, uint8_t *lds
   }
   }
   wait_dma();
+  if constexpr (KS > 1) asm volatile("" ::"v"(warm));
 
   if constexpr (KS > 1) {
     // The groups' partial sums meet in LDS (the pipelines are dead: after the barrier every copy has landed and every
