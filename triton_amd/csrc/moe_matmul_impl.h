@@ -117,30 +117,38 @@ TAMD_DEVICE bool locate_tile(const tamd_matmul_args &a, int grid_n, int64_t grid
   // A ragged launch is sized for the worst split of the rows over the experts (grid_total), about twice what a
   // balanced routing needs; the schedule's real entries come first and their number is block_offs[n_experts].  The
   // XCD ranges are cut from that number, read here, so that all eight XCDs share the real tiles; the rest exit.
+  // (the launchers keep a grid below 2^31 tiles: 32-bit unsigned arithmetic, whose divisions cost a third of the 64-bit ones)
+  uint32_t total = (uint32_t)grid_total;
+  const uint32_t gn = (uint32_t)grid_n;
   if (a.block_schedule && a.block_offs) {
-    const int64_t real_total = (int64_t)a.block_offs[a.n_experts] * grid_n;
-    grid_total = real_total < grid_total ? real_total : grid_total;
+    const uint64_t real_total = (uint64_t)(uint32_t)a.block_offs[a.n_experts] * gn;
+    total = real_total < total ? (uint32_t)real_total : total;
   }
-  const int64_t per_xcd = (grid_total + 7) / 8;
-  if ((int64_t)(blockIdx.x / 8) >= per_xcd) return false;
-  int64_t pid = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (pid >= grid_total) return false;
+  const uint32_t per_xcd = (total + 7) / 8;
+  const uint32_t bx = blockIdx.x;
+  if (bx / 8 >= per_xcd) return false;
+  const uint32_t pid = (bx % 8) * per_xcd + bx / 8;
+  if (pid >= total) return false;
   // Tiles are walked in groups of `group_m` row blocks: row block fastest inside a group, then the
   // column tile.  With many row blocks per expert the workgroups running together then share one
   // column tile of weights while the group's activation rows stay in L2; group_m = 1 is the plain
   // row-block-major order (right when an expert has only a block or two).
   int pid_m, pid_n;
   if (group_m > 1) {
-    const int grid_m = (int)(grid_total / grid_n);
-    const int64_t in_group = (int64_t)group_m * grid_n;
-    const int first_m = (int)(pid / in_group) * group_m;
-    const int size_m = grid_m - first_m < group_m ? grid_m - first_m : group_m;
-    const int r = (int)(pid - (pid / in_group) * in_group);
-    pid_m = first_m + r % size_m;
-    pid_n = r / size_m;
+    const uint32_t gm = (uint32_t)group_m;
+    const uint32_t grid_m = total / gn;
+    const uint32_t in_group = gm * gn;
+    const uint32_t gi = pid / in_group;
+    const uint32_t first_m = gi * gm;
+    const uint32_t size_m = grid_m - first_m < gm ? grid_m - first_m : gm;
+    const uint32_t r = pid - gi * in_group;
+    const uint32_t q = r / size_m;
+    pid_m = (int)(first_m + (r - q * size_m));
+    pid_n = (int)q;
   } else {
-    pid_m = (int)(pid / grid_n);
-    pid_n = (int)(pid - (int64_t)pid_m * grid_n);
+    const uint32_t q = pid / gn;
+    pid_m = (int)q;
+    pid_n = (int)(pid - q * gn);
   }
   t.n0 = pid_n * BLOCK_N;
   t.z = 0;
@@ -189,16 +197,18 @@ TAMD_DEVICE bool locate_tile_sorted(const tamd_matmul_args &a, int grid_n, int g
   constexpr int NB = 4;                              // row blocks per thread
   constexpr int NK = BLOCK_M <= 32 ? 1 : (BLOCK_M + EXTRA) / 32;  // largest fragment count of a tile
   const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  // (grids stay below 2^31 tiles: 32-bit unsigned arithmetic throughout, whose divisions are the cheap ones)
+  const uint32_t gn = (uint32_t)grid_n;
   const int x = blockIdx.x % 8, j = blockIdx.x / 8;
-  const int slot = j / grid_n, pid_n = j - slot * grid_n;
+  const int slot = (int)((uint32_t)j / gn), pid_n = j - slot * grid_n;
   const int p = slot * 8 + x;                        // position of this workgroup's row block in the sorted order
   const int n_real = a.block_offs[a.n_experts];
   // the same workgroup in schedule order: XCD x owns the tiles [x * per_xcd, (x + 1) * per_xcd)
-  const int64_t real_total = (int64_t)n_real * grid_n, per_xcd = (real_total + 7) / 8;
-  const int64_t plain_pid = (int64_t)x * per_xcd + j;
-  const bool plain_live = j < per_xcd && plain_pid < real_total;
+  const uint32_t real_total = (uint32_t)n_real * gn, per_xcd = (real_total + 7) / 8;
+  const uint32_t plain_pid = (uint32_t)x * per_xcd + (uint32_t)j;
+  const bool plain_live = (uint32_t)j < per_xcd && plain_pid < real_total;
   if (p >= n_real && !plain_live) return false;
-  const int plain_m = plain_live ? (int)(plain_pid / grid_n) : -1;
+  const int plain_m = plain_live ? (int)(plain_pid / gn) : -1;
   const int nb = (grid_m + 255) / 256;               // <= NB (checked by the launcher)
   int sched[NB], ssize[NB], soffs[NB], key[NB];
 #pragma unroll
@@ -278,7 +288,7 @@ TAMD_DEVICE bool locate_tile_sorted(const tamd_matmul_args &a, int grid_n, int g
   const int sc = res[sorted ? 0 : 4], slice_rows = res[sorted ? 1 : 5], start_m = res[sorted ? 2 : 6];
   __syncthreads();                                   // the scratch may be overwritten from here on
   if (!found || sc == -1) return false;
-  t.n0 = (sorted ? pid_n : (int)(plain_pid - (int64_t)plain_m * grid_n)) * BLOCK_N;
+  t.n0 = (sorted ? pid_n : (int)(plain_pid - (uint32_t)plain_m * gn)) * BLOCK_N;
   t.z = 0;
   t.expert = sc & 0xFFFF;
   t.start_m = start_m;
