@@ -202,20 +202,24 @@ TAMD_DEVICE bool locate_tile_sorted(const tamd_matmul_args &a, int grid_n, int g
   const int x = blockIdx.x % 8, j = blockIdx.x / 8;
   const int slot = (int)((uint32_t)j / gn), pid_n = j - slot * grid_n;
   const int p = slot * 8 + x;                        // position of this workgroup's row block in the sorted order
+  // The schedule entries are requested before anything waits for the number of real ones (entries past it hold -1, and
+  // the schedule is grid_m entries wide): one round trip to memory instead of two.
+  const int nb = (grid_m + 255) / 256;               // <= NB (checked by the launcher)
+  int sched[NB], ssize[NB], soffs[NB], key[NB];
+#pragma unroll
+  for (int u = 0; u < NB; ++u) {
+    const int b = u * 256 + tid;
+    sched[u] = (u < nb && b < grid_m) ? a.block_schedule[b] : -1;
+  }
   const int n_real = a.block_offs[a.n_experts];
+#pragma unroll
+  for (int u = 0; u < NB; ++u) sched[u] = u * 256 + tid < n_real ? sched[u] : -1;
   // the same workgroup in schedule order: XCD x owns the tiles [x * per_xcd, (x + 1) * per_xcd)
   const uint32_t real_total = (uint32_t)n_real * gn, per_xcd = (real_total + 7) / 8;
   const uint32_t plain_pid = (uint32_t)x * per_xcd + (uint32_t)j;
   const bool plain_live = (uint32_t)j < per_xcd && plain_pid < real_total;
   if (p >= n_real && !plain_live) return false;
   const int plain_m = plain_live ? (int)(plain_pid / gn) : -1;
-  const int nb = (grid_m + 255) / 256;               // <= NB (checked by the launcher)
-  int sched[NB], ssize[NB], soffs[NB], key[NB];
-#pragma unroll
-  for (int u = 0; u < NB; ++u) {
-    const int b = u * 256 + tid;
-    sched[u] = (u < nb && b < n_real) ? a.block_schedule[b] : -1;
-  }
 #pragma unroll
   for (int u = 0; u < NB; ++u) {
     const int e = sched[u] == -1 ? 0 : (sched[u] & 0xFFFF);

@@ -406,6 +406,11 @@ def matmul(a, b, bias, a_ragged_metadata: Optional[RaggedTensorMetadata] = None,
         args.block_schedule = md.block_schedule(flags.block_m).data_ptr()
         args.block_m = flags.block_m
         args.grid_m = RaggedTensorMetadata.n_blocks(md.n_slices, M, flags.block_m)
+        # the kernels read up to grid_m entries of the schedule: metadata made for fewer rows than the matmul has is a
+        # caller's mistake that must not become a read past the table
+        if args.grid_m > md.block_schedule(flags.block_m).shape[-1]:
+            raise ValueError(f"a_ragged_metadata was made for fewer rows than the matmul has ({M}): its block schedule "
+                             f"holds {md.block_schedule(flags.block_m).shape[-1]} entries, {args.grid_m} are needed")
     else:
         args.force_variant = flags.block_m if "block_m" in _opt_flags._constraints() else 0
     args.activation, args.act_alpha, args.act_limit, args.act_has_limit = act, act_alpha, act_limit, has_limit
