@@ -717,6 +717,21 @@ def test_block_layout_gives_the_same_bits(kind, device):
     assert torch.equal(y_strided.view(torch.int16), y_blocks.view(torch.int16))
 
 
+def test_metadata_made_for_fewer_rows_is_refused(device):
+    """The kernels read as many schedule entries as the matmul's row count can need: ragged metadata made for fewer rows
+    than the gathered activations have is refused on the host instead of being read past its end."""
+    torch.manual_seed(0)
+    E, K, N = 40, 64, 64
+    sizes = torch.ones(E, dtype=torch.int32)
+    md = make_ragged_tensor_metadata(sizes.to(device), E)           # 40 rows: at most 40 row blocks
+    M = 2000                                                         # the matmul is given 2000 rows
+    w = torch.randn(E, K, N) * 0.05
+    v, s, _, _ = quantize_w(w, device)
+    x = torch.randn(M, K).to(torch.bfloat16).to(device)
+    with pytest.raises(ValueError, match="fewer rows"):
+        matmul(x, v, None, md, precision_config=PrecisionConfig(b_mx_scale=s, b_microblock_size=32))
+
+
 # ---------------------------------------------------------------------------- K groups (few 32-row tiles)
 
 
