@@ -68,40 +68,47 @@ TAMD_DEVICE float fp8_byte(uint32_t word) {
   else return __builtin_amdgcn_cvt_f32_fp8((int)word, SEL);
 }
 
-template <int SS, int RING_>
+template <int SS, int RING_, int NCW = 4>
 struct StreamShape {
-  static constexpr int CODE_BYTES = 4 * SS * 1024;  // image of 16 columns' codes, padded to whole 1 KB copies
-  static constexpr int NSC = (SS + 1) / 2;          // 1 KB pieces of the scale image: 16 * K/32 bytes, or the whole
+  static constexpr int TS = NCW * SS;               // super steps (128 K) of the whole K range: NCW compute waves x SS
+  static constexpr int CODE_BYTES = TS * 1024;      // image of 16 columns' codes, padded to whole 1 KB copies
+  static constexpr int NSC = (TS + 7) / 8;          // 1 KB pieces of the scale image: 16 * K/32 bytes, or the whole
   static constexpr int SC_BYTES = NSC * 1024;       // pre-shuffled block of 32 columns (ceil(K/256)*8 * 32 bytes)
   static constexpr int BIAS_BYTES = 256;            // 16 bias values, one dword each
   static constexpr int STAGE = CODE_BYTES + SC_BYTES + BIAS_BYTES;
-  static constexpr int RED_BYTES = 2 * 4 * 1024;    // partial sums: 2 buffers x 4 waves x 16x16 floats
+  static constexpr int RED_BYTES = 2 * NCW * 1024;  // partial sums: 2 buffers x NCW waves x 16x16 floats
   static constexpr int RING = RING_;
-  static constexpr int DMA_PER_STAGE = 2 * SS + NSC;  // most copies one wave has per stage
+  static constexpr int DMA_PER_STAGE = TS / 2 + NSC;  // most copies one wave has per stage
   static constexpr int LDS = RING * STAGE + RED_BYTES;
   static_assert(RING >= 2 && (RING - 1) * DMA_PER_STAGE < 64, "ring does not fit the vmcnt counter");
 };
 
-// SS: super steps (4 e8m0 groups = 128 K each) per wave; covers K <= 512 * SS.  N is a multiple of 16.
+// SS: super steps (4 e8m0 groups = 128 K each) per compute wave; covers K <= 128 * NCW * SS.  N is a multiple of 16.
 //
-// 512 threads in three roles: waves 0-3 compute (LDS -> convert -> MFMA -> partial sums), waves 4-5
-// issue and await the copies, waves 6-7 finish and store the previous unit.  A wave that issues copies
+// Three roles: waves 0 .. NCW-1 compute (LDS -> convert -> MFMA -> partial sums), the next NC waves issue and await
+// the copies, the last two finish and store the previous unit.  A wave that issues copies
 // stalls whenever the memory pipeline is full; with nothing else to do it refills the pipeline the
 // moment there is room, and the stalls never delay MFMA work or stores.
+// NCW: compute waves (4 or 8) that split K between them.  The same kernel without its conversions and MFMAs runs the
+// decode shape in 144 instead of 159 us, so the compute waves' part of a unit is on the critical path; eight waves
+// halve each wave's part but were slower in all (171 us), and the launcher uses four.
 // A8 (1: float8_e4m3fn, 2: float8_e5m2; 0: rows of XDT): the activations are stored as fp8 (optionally with e8m0 block
 // scales per 32 K) and are expanded to
 // XDT when a row block's slice is loaded into registers -- exact, so the K loop is the same as for 16-bit rows.
-template <int XDT, int ACT, int SS, int RING, int A8>
-__global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
+// NC: copying waves (2 or 4).  A 1 KB copy holds the wave that issues it for about 110 cycles, so two copying waves
+// move at most 18 bytes per cycle and CU, and with the K of the decode shape (24 pieces of codes per unit) they were
+// what a unit waited for; four take a quarter of a unit's pieces each.
+template <int XDT, int ACT, int SS, int RING, int A8, int NC, int NCW>
+__global__ __launch_bounds__((NCW + NC + 2) * 64, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
   typedef Mma<XDT> M;
   typedef typename M::frag_t frag_t;
-  typedef StreamShape<SS, RING> S;
+  typedef StreamShape<SS, RING, NCW> S;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr uint32_t kOob = 0x7FFFFFFFu;
   constexpr bool SW = ACT == TAMD_ACT_SWIGLU;
   const int tid = threadIdx.x;
   const int wave8 = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
-  const int wave = wave8 & 3;  // index inside its group of four
+  const int wave = wave8;      // (compute waves: which part of K)
   const int K = a.K, N = a.N, G = K / 32;
   const uint32_t col_bytes = (uint32_t)(K / 2);
 
@@ -143,12 +150,12 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
   };
   float *red = (float *)(lds + S::RING * S::STAGE);
 
-  if (wave8 >= 6) {
+  if (wave8 >= NCW + NC) {
     // =========================================================================== finishing waves
     // 128 threads: thread -> (row er, column pair pc) of the 16x16 result of a unit; they read the four
     // partial sums one stage late, apply scale / bias / activation / gate weight and store.  These
     // waves never issue copies, so their loads and stores do not interfere with the copy counters.
-    const int ft = tid - 384;
+    const int ft = tid - (NCW + NC) * 64;
     const int er = ft / 8, pc = ft % 8;
     float flex = 1.0f;
     if (a.x_scale) flex *= *a.x_scale;
@@ -192,9 +199,13 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
       return clamp_out ? __builtin_fminf(__builtin_fmaxf(v, -out_max), out_max) : v;
     };
     auto finish = [&](int buf) {
-      const float *rbuf = red + buf * 1024 + red_idx;
-      const float s0 = (rbuf[0] + rbuf[256]) + (rbuf[512] + rbuf[768]);
-      const float s1 = (rbuf[4] + rbuf[260]) + (rbuf[516] + rbuf[772]);
+      const float *rbuf = red + buf * (NCW * 256) + red_idx;
+      float s0 = (rbuf[0] + rbuf[256]) + (rbuf[512] + rbuf[768]);
+      float s1 = (rbuf[4] + rbuf[260]) + (rbuf[516] + rbuf[772]);
+      if constexpr (NCW == 8) {
+        s0 += (rbuf[1024] + rbuf[1280]) + (rbuf[1536] + rbuf[1792]);
+        s1 += (rbuf[1028] + rbuf[1284]) + (rbuf[1540] + rbuf[1796]);
+      }
       const float v0 = (s0 * flex + p_bias0 * p_beta) * a.out_alpha;
       const float v1 = (s1 * flex + p_bias1 * p_beta) * a.out_alpha;
       if (p_dst < 0) return;
@@ -254,19 +265,20 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         atomicMax((unsigned int *)a.y_actual_scale, f32_to_bits(__builtin_fmaf(bits_to_f32(amax), 1.0f / out_max, 1.0e-30f)));
       }
     }
-  } else if (wave8 >= 4) {
+  } else if (wave8 >= NCW) {
     // =========================================================================== copying waves
     // Wave 4 requests the first half of a unit's code image and its scale image, wave 5 the second half
     // and the bias.  A wave that issues copies stalls whenever the memory pipeline is full, which is
     // exactly how these two keep it full; nothing else runs on them.
-    const int half = wave8 - 4;
+    const int half = wave8 - NCW;   // which part of a unit's code image this wave copies (0 .. NC - 1)
     const v4i_t rw = make_rsrc(a.w, kOob), rs = make_rsrc(a.w_mx_scale, kOob), rb = make_rsrc(a.bias, kOob);
     // empty descriptors (no records: every lane out of range) for copies past the end of the range,
     // issued so that the count of outstanding copies per stage never changes
     const v4i_t rw0 = make_rsrc(a.w, 0), rs0 = make_rsrc(a.w_mx_scale, 0), rb0 = make_rsrc(a.bias, 0);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const int bias_esz = a.bias_dtype == TAMD_F32 ? 4 : 2;
-    constexpr int NP = 2 * SS;  // code pieces (1 KB) per copying wave
+    constexpr int NP = S::TS / NC;  // code pieces (1 KB) per copying wave
+    static_assert(S::TS % NC == 0, "the copying waves take equal parts of a unit's code image");
     // per-lane source offsets never change: a unit's codes, scales and bias are linear images
     uint32_t w_voff[NP];
 #pragma unroll
@@ -282,7 +294,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
 #pragma unroll
       for (int q = 0; q < S::NSC; ++q) x_voff[q] = q * 1024u + lane * 16u < sc_unit_bytes ? q * 1024u + lane * 16u : kOob;
     } else {
-      x_voff[0] = (a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
+      x_voff[0] = (half == 1 && a.bias != nullptr && lane < 16) ? (uint32_t)(lane * bias_esz) : kOob;
 #pragma unroll
       for (int q = 1; q < S::NSC; ++q) x_voff[q] = kOob;
     }
@@ -330,7 +342,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         const uint32_t so = i_sbase + (cdna4 ? (uint32_t)(i_cg >> 1) : (uint32_t)i_cg) * sc_unit_bytes;
 #pragma unroll
         for (int q = 0; q < S::NSC; ++q) dma16(live ? rs : rs0, sb + S::CODE_BYTES + q * 1024, x_voff[q], so);
-      } else {
+      } else if (half == 1) {
         const uint32_t dst = sb + S::CODE_BYTES + S::SC_BYTES;
         if (bias_esz == 4) dma4(live ? rb : rb0, dst, x_voff[0], i_bbase);
         else dma2(live ? rb : rb0, dst, x_voff[0], i_bbase);
@@ -349,7 +361,8 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
     for (int s = 0; s < total_stages; ++s) {
       // copies complete in order: once at most RING - 2 stages' worth are outstanding, stage s has landed
       if (half == 0) wait_vmcnt<(S::RING - 2) * (NP + S::NSC)>();
-      else wait_vmcnt<(S::RING - 2) * (NP + 1)>();
+      else if (half == 1) wait_vmcnt<(S::RING - 2) * (NP + 1)>();
+      else wait_vmcnt<(S::RING - 2) * NP>();
       __syncthreads();  // publishes stage s; every wave is done with stage s - 1, whose slot is refilled now
       issue(i_slot);
       i_slot = i_slot + 1 == S::RING ? 0 : i_slot + 1;
@@ -462,7 +475,7 @@ __global__ __launch_bounds__(512, 1) void mm_stream16_kernel(tamd_matmul_args a,
         acc2 = Mma16<XDT>::mma(areg[j * 4 + 2], M::expand(raw[j].z, sc), acc2);
         acc3 = Mma16<XDT>::mma(areg[j * 4 + 3], M::expand(raw[j].w, sc), acc3);
       }
-      *(f32x4_t *)(red + (s & 1) * 1024 + wave * 256 + lane * 4) = (acc0 + acc1) + (acc2 + acc3);
+      *(f32x4_t *)(red + (s & 1) * (NCW * 256) + wave * 256 + lane * 4) = (acc0 + acc1) + (acc2 + acc3);
       slot = slot + 1 == S::RING ? 0 : slot + 1;
     }
     __syncthreads();
@@ -491,9 +504,13 @@ inline bool stream16_applicable(const tamd_matmul_args &a) {
   return true;
 }
 
-template <int XDT, int ACT, int SS, int A8>
+template <int XDT, int ACT, int SS, int A8, int NCW>
 int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
-  constexpr int RING_FIT = (156 * 1024 - 8192) / (4 * SS * 1024 + (SS + 1) / 2 * 1024 + 256);
+  constexpr int TS = NCW * SS;
+  // four copying waves where the registers allow three or four waves per SIMD (the kernels that expand fp8 rows keep a
+  // wave's whole slice of the rows in registers twice over while they convert it)
+  constexpr int NC = NCW * 64 + 6 * 64 <= 640 && (A8 == 0 ? SS <= 6 : SS <= 4) ? 4 : 2;
+  constexpr int RING_FIT = (156 * 1024 - 2 * NCW * 1024) / (TS * 1024 + (TS + 7) / 8 * 1024 + 256);
   constexpr int RING = RING_FIT > 6 ? 6 : RING_FIT;
   const int n_cg = (a.N + 15) / 16;
   const int64_t upper = (int64_t)grid_m * n_cg;
@@ -501,19 +518,21 @@ int launch_stream16_ss(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
   int cus = 0;
   if (int rc = cu_count(cus)) return rc;
   const int wgs = (int)(upper < cus ? upper : cus);
-  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, A8>;
+  auto kern = mm_stream16_kernel<XDT, ACT, SS, RING, A8, NC, NCW>;
   if (int rc = raise_lds_limit_once((const void *)kern)) return rc;
-  kern<<<dim3((unsigned)wgs), 512, StreamShape<SS, RING>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
+  kern<<<dim3((unsigned)wgs), (NCW + NC + 2) * 64, StreamShape<SS, RING, NCW>::LDS, st>>>(a, n_cg, a.block_schedule ? 0 : grid_m);
   return launch_status();
 }
 
 template <int XDT, int ACT, int A8 = 0>
 int launch_stream16(const tamd_matmul_args &a, int grid_m, hipStream_t st) {
+  // four compute waves: with eight (each wave half the conversions and MFMAs of a unit, fourteen waves at the unit's
+  // barrier, eight partial sums to add) the decode shape ran 171 us instead of 159
   const int ss = (a.K / 32 + 15) / 16;  // super steps per wave
-  if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2, A8>(a, grid_m, st);
-  if (ss <= 4) return launch_stream16_ss<XDT, ACT, 4, A8>(a, grid_m, st);
-  if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6, A8>(a, grid_m, st);
-  return launch_stream16_ss<XDT, ACT, 8, A8>(a, grid_m, st);
+  if (ss <= 2) return launch_stream16_ss<XDT, ACT, 2, A8, 4>(a, grid_m, st);
+  if (ss <= 4) return launch_stream16_ss<XDT, ACT, 4, A8, 4>(a, grid_m, st);
+  if (ss <= 6) return launch_stream16_ss<XDT, ACT, 6, A8, 4>(a, grid_m, st);
+  return launch_stream16_ss<XDT, ACT, 8, A8, 4>(a, grid_m, st);
 }
 
 // The streaming kernels of one activation type live in a translation unit of their own (moe_matmul_stream_*.hip).
