@@ -27,7 +27,7 @@ KINDS = ["bf16", "f16", "e4m3", "e5m2", "mxfp8"]
 def make_case(seed):
     rng = random.Random(seed)
     c = dict(seed=seed)
-    c["kind"] = KINDS[seed % len(KINDS)]
+    c["kind"] = "mxfp4" if seed % 11 == 10 else KINDS[seed % len(KINDS)]   # MXFP4 rows: every eleventh case
     c["E"] = rng.choice([1, 2, 5, 9])
     c["K"] = 32 * rng.choice([1, 2, 3, 5, 10, 13, 32, 45] + ([90, 128, 129, 160, 256] if os.environ.get("TAMD_SWEEP_LONG_K") else []))
     c["N"] = 2 * rng.choice([8, 16, 33, 100, 128, 131, 264, 300])
@@ -98,14 +98,15 @@ def test_sweep(seed, device):
         out_dtype = c["out"]
     else:
         x0 = x0 * torch.exp(torch.randn(n_src, K // 32).repeat_interleave(32, dim=1))
-        xv, xs = downcast_to_mxfp(x0.to(device), torch.float8_e4m3fn, axis=-1)
-        rq, rxs = downcast_to_mxfp_ref(x0, torch.float8_e4m3fn, axis=-1)
+        vdt = torch.uint8 if kind == "mxfp4" else torch.float8_e4m3fn   # packed e2m1 codes or e4m3 values
+        xv, xs = downcast_to_mxfp(x0.to(device), vdt, axis=-1)
+        rq, rxs = downcast_to_mxfp_ref(x0, vdt, axis=-1)
         assert torch.equal(xv.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs.cpu(), rxs)
         if gather is None:
             xv, xs, rq, rxs = xv[:M], xs[:M], rq[:M], rxs[:M]
         xdev = xv
         pc = PrecisionConfig(a_mx_scale=xs, a_microblock_size=32, b_mx_scale=sc, b_microblock_size=32, out_dtype=c["out"])
-        ref = MR.matmul_ref(rq, rv, bias, a_mx_scale=rxs, **kw)
+        ref = MR.matmul_ref(rq.contiguous(), rv, bias, a_mx_scale=rxs.contiguous(), **kw)
         out_dtype = c["out"]
     dev = lambda t: None if t is None else t.to(device)
     md = make_ragged_tensor_metadata(sizes.to(device), M)
