@@ -1448,7 +1448,7 @@ inline int dense_block_m(const tamd_matmul_args &a) {
   return 16;  // too few tiles either way: the smallest block gives the most
 }
 // A dense / batched problem of 161 to 256 rows whose 32-row tiles number at most half the CUs and whose K holds at
-// least eight 128-K pairs: faster as 32-row tiles with four K groups each (256 x 2048 x 4096: 14.6 us) than as 16-row
+// least eight 128-K pairs: faster as 32-row tiles with four K groups each (256 x 2048 x 4096: 13.8 us) than as 16-row
 // blocks through the streaming kernel (22 us), which is what problems of fewer rows take.
 inline bool dense_prefers_k_groups(const tamd_matmul_args &a) {
   if (is_fp8(a.x_dtype) || a.M <= 160 || a.M > 256 || (a.K + KB - 1) / KB < 8) return false;

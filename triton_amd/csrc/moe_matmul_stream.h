@@ -10,7 +10,7 @@
 //   * one workgroup per CU walks a contiguous range of units, cut from the number of real row blocks
 //     read on the device (block_offs[n_experts]), so consecutive units continue the same linear
 //     stream and the padding of the block schedule costs nothing;
-//   * two waves copy, four compute, two finish.  The copying waves send the runs HBM -> LDS by DMA
+//   * two or four waves copy, four compute, two finish.  The copying waves send the runs HBM -> LDS by DMA
 //     (buffer_load ... lds) as they lie in memory, through a ring of stages filled several units
 //     ahead (about 100 KB in flight per CU); every per-unit operand, bias included, travels in that
 //     stream so that no other load ever drains it;
@@ -90,14 +90,14 @@ struct StreamShape {
 // stalls whenever the memory pipeline is full; with nothing else to do it refills the pipeline the
 // moment there is room, and the stalls never delay MFMA work or stores.
 // NCW: compute waves (4 or 8) that split K between them.  The same kernel without its conversions and MFMAs runs the
-// decode shape in 144 instead of 159 us, so the compute waves' part of a unit is on the critical path; eight waves
-// halve each wave's part but were slower in all (171 us), and the launcher uses four.
+// decode shape in 144 instead of 159 us; eight waves halve each wave's part of a unit but were slower in all (171 us:
+// fourteen waves at the unit's barrier, eight partial sums to add), and the launcher uses four.
 // A8 (1: float8_e4m3fn, 2: float8_e5m2; 0: rows of XDT): the activations are stored as fp8 (optionally with e8m0 block
 // scales per 32 K) and are expanded to
 // XDT when a row block's slice is loaded into registers -- exact, so the K loop is the same as for 16-bit rows.
 // NC: copying waves (2 or 4).  A 1 KB copy holds the wave that issues it for about 110 cycles, so two copying waves
-// move at most 18 bytes per cycle and CU, and with the K of the decode shape (24 pieces of codes per unit) they were
-// what a unit waited for; four take a quarter of a unit's pieces each.
+// move at most 18 bytes per cycle and CU and, with the K of the decode shape (24 pieces of codes per unit), spend
+// most of a unit issuing; four take a quarter of a unit's pieces each (decode shape: 161 -> 158 us).
 template <int XDT, int ACT, int SS, int RING, int A8, int NC, int NCW>
 __global__ __launch_bounds__((NCW + NC + 2) * 64, 1) void mm_stream16_kernel(tamd_matmul_args a, int n_cg, int dense_blocks) {
   typedef Mma<XDT> M;
